@@ -1,0 +1,145 @@
+/* turbofft.h -- C ABI of libturbofft_hip.so, the MI355X (gfx950) batched
+ * radix-2 C2C forward FFT engine.
+ *
+ * The reference (shixun404/TurboFFT) has no library API: its two seams are
+ * the kernel ABI `fft_radix_2<T,logN,dim,ft,err>(in,out,twiddle,checksum_DFT,
+ * BS,thread_bs)` selected from a function-pointer table
+ * (include/TurboFFT.h:22-25, include/TurboFFT_radix_2_template.h:1-3,
+ * launched at main.cu:48) and the `turbofft` executable with its flags
+ * (include/utils/CommandLineParser.h:26-45).  Every entry point below names
+ * the reference code it stands in for.  Plain pointers and sizes only; all
+ * functions return 0 on success and a negative code on error, with a message
+ * available from turbofft_last_error().  Nothing in the library exits the
+ * process or falls back to a CPU computation.
+ *
+ * Data layout (main.cu:99-101, initializeData.h): interleaved {re,im},
+ * batch-major x[b*N + n]; the result is out-of-place, natural order, same
+ * shape.  `in` is never written.  When the plan uses more than one launch
+ * `out` must hold 2*N*bs elements (initializeData.h:21, main.cu:11-12); the
+ * transform is left in out[0 .. N*bs), the second half is workspace.
+ */
+#ifndef TURBOFFT_H
+#define TURBOFFT_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct turbofft_plan turbofft_plan_t;
+
+#define TURBOFFT_FP32 0   /* float2,  --datatype 0 (CommandLineParser.h:75-77) */
+#define TURBOFFT_FP64 1   /* double2, --datatype 1 */
+
+#define TURBOFFT_OK            0
+#define TURBOFFT_EINVAL       -1  /* bad argument                                   */
+#define TURBOFFT_ENOPLAN      -2  /* no plan row / no compiled kernel for the shape */
+#define TURBOFFT_EHIP         -3  /* a HIP runtime call failed                       */
+#define TURBOFFT_ENOMEM       -4
+
+/* Last error message of the calling thread ("" if none). */
+const char* turbofft_last_error(void);
+
+/* Create a plan for N = 2^logN.
+ * Stands in for: load_parameters + params[logN] (main.cu:83, readCSV.h:14-33),
+ * the TurboFFT_Kernel_Entry lookup (TurboFFT.h:22-25), the launch-geometry
+ * and shared-memory attribute setup of test_turbofft (main.cu:21-42), the
+ * twiddle table of initializeData (initializeData.h:31-37) and the DFT
+ * checksum table (abft.h:21-61, main.cu:85-93).
+ *   datatype   TURBOFFT_FP32 / TURBOFFT_FP64
+ *   if_ft      1: fault-tolerant kernels (fused two-sided checksums)
+ *   if_err     1: inject errors with the reference cadence and correct them
+ *              (implies if_ft, CommandLineParser.h:66-68)
+ *   thread_bs  tiles per block = checksum group size (--thread_bs)
+ *   param_csv  plan CSV in the reference's 11-column format, row index ==
+ *              logN; NULL selects the built-in gfx950 table.
+ * Returns NULL on error. */
+turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_err,
+                                      int thread_bs, const char* param_csv);
+
+/* Stands in for the cudaFree calls at the end of TurboFFT_main (main.cu:130-132). */
+void turbofft_plan_destroy(turbofft_plan_t* plan);
+
+/* Asynchronous transform of `bs` length-N sequences on `stream`
+ * (a hipStream_t; NULL = the null stream).  Device pointers.
+ * Stands in for the launch loop of test_turbofft (main.cu:46-49, 55-58). */
+int turbofft_exec(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs, void* stream);
+
+/* Same, from and to host memory (allocates device buffers, copies, runs,
+ * synchronises, frees).  Stands in for initializeData's H2D copy plus the
+ * D2H copy at main.cu:72. */
+int turbofft_exec_host(turbofft_plan_t* plan, const void* in_h, void* out_h, long long bs);
+
+/* Timed runs with HIP events on `stream`: `warmup` untimed executions, then
+ * `reps` timed ones with no host synchronisation in between; *ms_per_exec
+ * receives the mean.  Stands in for the timing of test_turbofft
+ * (main.cu:44-67; the reference synchronises after every launch, this does not). */
+int turbofft_time(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
+                  int warmup, int reps, void* stream, float* ms_per_exec);
+
+/* Plan description: launches, per-launch log2 size, BS, n, dynamic LDS bytes,
+ * threads per block (the CSV row, main.cu:8-9,22-27). */
+int turbofft_plan_info(const turbofft_plan_t* plan, int* launches, int logNi[3], int BSi[3],
+                       int ni[3], size_t lds_bytes[3], int threads[3]);
+
+/* Grid size of launch `launch` for `bs` transforms (main.cu:32). */
+long long turbofft_plan_grid(const turbofft_plan_t* plan, int launch, long long bs);
+
+/* Tile interleave distance of launch `launch` (the reference's tb_gap,
+ * fft_codegen.py:216-218, with resident blocks measured on this device). */
+int turbofft_plan_tb_gap(const turbofft_plan_t* plan, int launch);
+/* Override it (tests use this to make groups reproducible). */
+int turbofft_plan_set_tb_gap(turbofft_plan_t* plan, int launch, int tb_gap);
+
+/* ---- fault tolerance (no counterpart API in the reference; its generator
+ * bakes these into the kernel text: fft_codegen.py:412-415, 495, 714-719) ---- */
+
+/* Detection rule |delta| / (err_smoothing + |mag|) > err_threshold. */
+int turbofft_set_ft_params(turbofft_plan_t* plan, double err_smoothing, double err_threshold, int correct);
+
+/* Error injection for the launch `launch` (-1 = last, the reference's choice):
+ *   mode 0  none
+ *   mode 1  reference cadence: in every `every`-th block, the tile with
+ *           cnt == block % thread_bs + 1 gets `mag` added to re of element
+ *           (s, m) after the input checksum (s = m = 0 in the reference)
+ *   mode 2  tiles with tile % every == tile_phase                              */
+int turbofft_set_injection(turbofft_plan_t* plan, int mode, int launch, int every,
+                           long long tile_phase, int s, int m, double mag);
+
+/* Counters accumulated since the last reset: groups checked, detected,
+ * corrected, uncorrectable (located tile out of range); flagged[2*i] = launch,
+ * flagged[2*i+1] = tile (-1 if not locatable), up to `cap` pairs; *nflagged
+ * receives the number recorded.  Synchronises the device. */
+int turbofft_get_ft_counters(turbofft_plan_t* plan, unsigned long long* checked,
+                             unsigned long long* detected, unsigned long long* corrected,
+                             unsigned long long* uncorrectable, long long* flagged, int cap,
+                             int* nflagged);
+int turbofft_reset_ft_counters(turbofft_plan_t* plan);
+
+/* ---- host tables (no device needed) ---- */
+
+/* tw[c-1+m] = exp(-2 pi i m / c), c = 1,2,4..N; 2N-1 entries of T
+ * (initializeData.h:31-37). */
+int turbofft_build_twiddle_table(int datatype, long long N, void* out);
+
+/* c_N[i] = sum_j W_N^{ij} r[j%3], N entries of T (abft.h:21-61).
+ * mode 0: exact angles; mode 1: the reference's float-rounded angles. */
+int turbofft_build_checksum_vector(int datatype, long long N, int mode, void* out);
+
+/* Built-in gfx950 plan row for logN: writes the 11 CSV columns. */
+int turbofft_builtin_plan_row(int datatype, int logN, int row[11]);
+
+/* Number of compiled kernels and their names (registry introspection; the
+ * role of test.py, which prints the reference's dispatch tables). */
+int turbofft_kernel_count(void);
+const char* turbofft_kernel_name(int i);
+
+/* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
+ * flags and output lines.  Returns the process exit code. */
+int turbofft_main(int argc, char** argv);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

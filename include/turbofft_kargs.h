@@ -1,0 +1,56 @@
+/* Kernel argument block shared by the host driver and every generated kernel.
+ *
+ * Plain C, passed by value as the last kernel argument (it lands in SGPRs).
+ * It replaces the reference kernel ABI's trailing `int BS, int thread_bs`
+ * (include/TurboFFT_radix_2_template.h:1-3, fft_codegen.py:207-211): the
+ * reference bakes every stride into the generated text, these kernels take the
+ * launch geometry at run time so one kernel per (type, kind, Ni, BS, n) serves
+ * every logN that uses that tile shape.
+ */
+#ifndef TURBOFFT_KARGS_H
+#define TURBOFFT_KARGS_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tfft_ft_args {
+    const void* cksum;            /* c_Ni, Ni entries of T (input-side encoding vector)   */
+    unsigned long long* counters; /* [0]=groups checked [1]=detected [2]=corrected
+                                     [3]=uncorrectable  [4]=flagged-list length            */
+    long long* flagged;           /* flagged tile ids: flagged[2*i]=launch, [2*i+1]=tile   */
+    int flagged_cap;
+    int launch;                   /* launch index written into `flagged`                   */
+    int correct;                  /* 1: recompute the located tile (the if_err=1 variants) */
+    int inj_mode;                 /* 0 none; 1 reference cadence (tile cnt == block %
+                                     thread_bs + 1 of every `inj_every`-th block);
+                                     2 host-chosen tile(s): tile % inj_every == inj_tile   */
+    int inj_every;
+    long long inj_tile;
+    int inj_s;                    /* sub-FFT inside the tile                               */
+    int inj_m;                    /* element of that sub-FFT                               */
+    double inj_mag;               /* added to the real part after the input checksum       */
+    double err_smoothing;         /* |delta| / (err_smoothing + |mag|) > err_threshold     */
+    double err_threshold;
+} tfft_ft_args;
+
+typedef struct tfft_kargs {
+    long long ntiles;     /* tiles in this launch (a tile = BS sub-FFTs of length Ni)      */
+    long long nrows;      /* row1: number of transforms (guards a ragged last tile)        */
+    int thread_bs;        /* tiles a block processes in sequence (one checksum group)      */
+    int tb_gap;           /* interleave distance between a block's consecutive tiles       */
+    int log_ncols;        /* col : log2(contiguous columns per outer block)                */
+    int logQ;             /* rowT: rows of a transform are q + Q*s', q<Q, s'<C             */
+    int logC;
+    int logN;             /* rowT: log2 of the whole transform                             */
+    int tw_lo_bits;       /* col : W^e = tw_hi[e >> lo_bits] * tw_lo[e & mask]             */
+    int pad0;
+    const void* tw_hi;
+    const void* tw_lo;
+    tfft_ft_args ft;
+} tfft_kargs;
+
+#ifdef __cplusplus
+}
+#endif
+#endif

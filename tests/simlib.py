@@ -1,0 +1,103 @@
+"""Test helper: build and run the CPU lock-step flavour of generated kernels.
+
+The generator prints every kernel as barrier-separated phases; with
+-DTFFT_SIM the same text runs on the CPU, one phase for all threads at a
+time, with bounds-checked accessors.  This validates the generator's index
+algebra, LDS layouts and barrier placement here, where there is no GPU.
+"""
+import ctypes as C
+import hashlib
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+
+from turbofft_amd.codegen.fft_codegen import KernelSpec, generate_source
+from turbofft_amd.codegen.plan import KernelKey
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_CACHE = os.path.join(tempfile.gettempdir(), "tfft_sim_cache")
+
+
+class FtArgs(C.Structure):
+    _fields_ = [("cksum", C.c_void_p), ("counters", C.c_void_p), ("flagged", C.c_void_p),
+                ("flagged_cap", C.c_int), ("launch", C.c_int), ("correct", C.c_int),
+                ("inj_mode", C.c_int), ("inj_every", C.c_int), ("inj_tile", C.c_longlong),
+                ("inj_s", C.c_int), ("inj_m", C.c_int), ("inj_mag", C.c_double),
+                ("err_smoothing", C.c_double), ("err_threshold", C.c_double)]
+
+
+class KArgs(C.Structure):
+    _fields_ = [("ntiles", C.c_longlong), ("nrows", C.c_longlong), ("thread_bs", C.c_int),
+                ("tb_gap", C.c_int), ("log_ncols", C.c_int), ("logQ", C.c_int), ("logC", C.c_int),
+                ("logN", C.c_int), ("tw_lo_bits", C.c_int), ("pad0", C.c_int),
+                ("tw_hi", C.c_void_p), ("tw_lo", C.c_void_p), ("ft", FtArgs)]
+
+
+def ctype_of(dtype):
+    return np.complex64 if dtype == "float2" else np.complex128
+
+
+def twiddle_table(N, dtype):
+    out = np.empty(2 * N - 1, dtype=np.complex128)
+    c = 1
+    while c <= N:
+        out[c - 1:2 * c - 1] = np.exp(-2j * np.pi * np.arange(c) / c)
+        c *= 2
+    return out.astype(ctype_of(dtype))
+
+
+def build_sim(spec: KernelSpec):
+    src = generate_source([spec], True).replace(
+        '#include "../tfft_device.h"', f'#include "{ROOT}/turbofft_amd/csrc/tfft_device.h"')
+    src += "\ntfft_sim_bounds_t tfft_sim_bounds; long long tfft_sim_errors = 0;\n"
+    src += 'extern "C" long long tfft_sim_error_count() { return tfft_sim_errors; }\n'
+    h = hashlib.sha1(src.encode()).hexdigest()[:16]
+    os.makedirs(_CACHE, exist_ok=True)
+    so = os.path.join(_CACHE, f"{spec.name}_{h}.so")
+    if not os.path.exists(so):
+        cpp = so[:-3] + ".cpp"
+        with open(cpp, "w") as f:
+            f.write(src)
+        subprocess.check_call(["g++", "-O1", "-shared", "-fPIC", "-o", so, cpp])
+    return C.CDLL(so)
+
+
+def run_sim(spec: KernelSpec, x_in: np.ndarray, out_elems: int, kargs: KArgs, grid: int,
+            tw: np.ndarray, twhi=None, twlo=None, ck=None):
+    lib = build_sim(spec)
+    fn = getattr(lib, spec.name + "_sim")
+    ct = ctype_of(spec.T2)
+    x_in = np.ascontiguousarray(x_in, dtype=ct).ravel()
+    out = np.full(out_elems, np.nan + 1j * np.nan, dtype=ct)
+    tw = np.ascontiguousarray(tw, dtype=ct)
+    keep = [x_in, out, tw]
+    lim = np.zeros(6, dtype=np.int64)
+    lim[0], lim[1], lim[2] = x_in.size, out.size, tw.size
+    if twhi is not None:
+        twhi = np.ascontiguousarray(twhi, dtype=ct); twlo = np.ascontiguousarray(twlo, dtype=ct)
+        kargs.tw_hi = twhi.ctypes.data; kargs.tw_lo = twlo.ctypes.data
+        lim[3], lim[4] = twhi.size, twlo.size
+        keep += [twhi, twlo]
+    if ck is not None:
+        ck = np.ascontiguousarray(ck, dtype=ct)
+        kargs.ft.cksum = ck.ctypes.data
+        lim[5] = ck.size
+        keep.append(ck)
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(KArgs), C.c_longlong, C.c_void_p]
+    fn.restype = None
+    fn(x_in.ctypes.data, out.ctypes.data, tw.ctypes.data, C.byref(kargs), grid, lim.ctypes.data)
+    lib.tfft_sim_error_count.restype = C.c_longlong
+    errs = lib.tfft_sim_error_count()
+    assert errs == 0, f"{errs} out-of-bounds accesses in {spec.name}"
+    return out
+
+
+def split_tables(logL, dtype):
+    """Two-level table for W_(2^L)^e: hi[h] = W^(h << lo_bits), lo[l] = W^l."""
+    lo_bits = (logL + 1) // 2
+    L = 1 << logL
+    hi = np.exp(-2j * np.pi * (np.arange(1 << (logL - lo_bits)) << lo_bits) / L)
+    lo = np.exp(-2j * np.pi * np.arange(1 << lo_bits) / L)
+    return lo_bits, hi.astype(ctype_of(dtype)), lo.astype(ctype_of(dtype))

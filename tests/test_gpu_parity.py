@@ -1,0 +1,166 @@
+"""GPU parity: the gfx950 kernels, called through the C ABI, against the fp64
+numpy DFT on the same seeded inputs.  Tolerances are the ones the task states:
+rel-L2 <= 1e-5*log2N (fp32), <= 1e-13*log2N (fp64)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import turbofft_amd
+from oracle import turbofft_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _torch():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    return torch
+
+
+def cdtype(dt):
+    return np.complex64 if dt == "float2" else np.complex128
+
+
+def make(bs, N, dt, seed=0, normal=False):
+    rng = np.random.default_rng(seed)
+    if normal:
+        x = rng.standard_normal((bs, N)) + 1j * rng.standard_normal((bs, N))
+    else:
+        x = rng.uniform(-1, 1, (bs, N)) + 1j * rng.uniform(-1, 1, (bs, N))
+    return x.astype(cdtype(dt))
+
+
+def gpu_fft(plan, x):
+    torch = _torch()
+    print(f"[case] logN={plan.logN} dt={plan.datatype} bs={x.shape[0]} launches={plan.launches} "
+          f"Ni={plan.logNi} BS={plan.BS} n={plan.n}", flush=True)
+    y = plan.fft(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def test_config1_fp64_2p10_batch16():
+    # BASELINE config 1: fp64, N=2^10, batch 16, U[-1,1) seed 0, single launch n=8
+    plan = turbofft_amd.TurboFFT(10, "double2")
+    assert plan.launches == 1 and plan.n == [8]
+    x = make(16, 1024, "double2", 0)
+    y = gpu_fft(plan, x)
+    assert O.rel_l2(y, O.fft_ref(x)) <= 1e-13 * 10
+
+
+@pytest.mark.parametrize("dt", ["float2", "double2"])
+@pytest.mark.parametrize("logN", list(range(1, 14)))
+def test_single_launch_sizes(dt, logN):
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    BS = plan.BS[0] if plan.launches == 1 else 1
+    bs = 3 * BS + max(1, BS // 2)              # ragged last tile
+    x = make(bs, 1 << logN, dt, logN)
+    y = gpu_fft(plan, x)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    # every transform individually (a wrong row in a tile must not hide in the norm)
+    ref = O.fft_ref(x)
+    for b in range(bs):
+        assert O.rel_l2(y[b], ref[b]) <= O.tolerance(dt, logN)
+
+
+@pytest.mark.parametrize("dt", ["float2", "double2"])
+@pytest.mark.parametrize("logN", list(range(14, 25)))
+def test_multi_launch_sizes(dt, logN):
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    bs = 3 if logN <= 20 else 1
+    x = make(bs, 1 << logN, dt, logN, normal=True)
+    y = gpu_fft(plan, x)
+    ref = O.fft_ref(x)
+    for b in range(bs):
+        assert O.rel_l2(y[b], ref[b]) <= O.tolerance(dt, logN)
+
+
+@pytest.mark.parametrize("dt,logN", [("float2", 13), ("double2", 15), ("float2", 24), ("double2", 20)])
+def test_closed_forms(dt, logN):
+    # impulse at n0 -> W^{n0 k} in natural order; constant -> N delta_0
+    N = 1 << logN
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    n0 = 12345 % N
+    x = np.zeros((2, N), cdtype(dt))
+    x[0, n0] = 1
+    x[1, :] = 1
+    y = gpu_fft(plan, x)
+    k = np.arange(N)
+    ref0 = np.exp(-2j * np.pi * ((n0 * k) % N) / N)
+    assert O.rel_l2(y[0], ref0) <= O.tolerance(dt, logN)
+    ref1 = np.zeros(N, complex); ref1[0] = N
+    assert np.max(np.abs(y[1] - ref1)) <= O.tolerance(dt, logN) * N
+
+
+def test_thread_bs_does_not_change_results():
+    x = make(64, 1 << 12, "float2", 3)
+    a = gpu_fft(turbofft_amd.TurboFFT(12, "float2", thread_bs=1), x)
+    b = gpu_fft(turbofft_amd.TurboFFT(12, "float2", thread_bs=5), x)
+    assert np.array_equal(a, b)
+
+
+def test_exec_host_matches_device_path():
+    x = make(8, 1 << 15, "double2", 4)
+    plan = turbofft_amd.TurboFFT(15, "double2")
+    a = plan.fft_host(x)
+    b = gpu_fft(plan, x)
+    assert np.array_equal(a, b)
+    assert O.rel_l2(a, O.fft_ref(x)) <= O.tolerance("double2", 15)
+
+
+def test_empty_batch_and_bad_shapes():
+    torch = _torch()
+    plan = turbofft_amd.TurboFFT(10, "float2")
+    plan.exec(0, 0, 0)                                   # bs = 0 is a no-op
+    with pytest.raises(ValueError):
+        plan.fft(torch.zeros((2, 512), dtype=torch.complex64, device="cuda"))
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        turbofft_amd.TurboFFT(30, "float2")              # no plan row
+
+
+def test_input_is_not_modified():
+    torch = _torch()
+    x = make(4, 1 << 16, "float2", 5)
+    xd = torch.from_numpy(x).cuda()
+    plan = turbofft_amd.TurboFFT(16, "float2")
+    plan.fft(xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(xd.cpu().numpy(), x)
+
+
+def test_config2_full_size_fp32_2p13():
+    # BASELINE config 2 at full size (2^28 points): sampled batches against the oracle,
+    # plus linearity of the whole batch as a size-independent property
+    torch = _torch()
+    logN, bs = 13, 1 << 15
+    N = 1 << logN
+    plan = turbofft_amd.TurboFFT(logN, "float2")
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = (torch.rand((bs, N, 2), generator=g, device="cuda", dtype=torch.float32) * 2 - 1)
+    x = torch.view_as_complex(x)
+    y = plan.fft(x)
+    torch.cuda.synchronize()
+    idx = [0, 1, 777, bs // 2, bs - 1]
+    xs = x[idx].cpu().numpy()
+    ys = y[idx].cpu().numpy()
+    ref = O.fft_ref(xs)
+    for i in range(len(idx)):
+        assert O.rel_l2(ys[i], ref[i]) <= O.tolerance("float2", logN)
+    # Parseval over the whole set: sum |X|^2 = N sum |x|^2
+    ex = float((x.real.double() ** 2 + x.imag.double() ** 2).sum())
+    ey = float((y.real.double() ** 2 + y.imag.double() ** 2).sum())
+    assert abs(ey / (N * ex) - 1) < 1e-5
+
+
+def test_cli_verify_mode():
+    for dt, logN, bs in ((1, 10, 16), (0, 13, 4), (1, 15, 2)):
+        r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "0", "--if_verify", "1", "--logN", str(logN),
+                            "--bs", str(bs), "--bs_end", str(bs), "--datatype", str(dt)],
+                           capture_output=True, text=True, timeout=120)
+        print(r.stdout, r.stderr, flush=True)
+        assert r.returncode == 0
+        assert "Compare begin." in r.stdout and "Compare finished." in r.stdout
+        assert "Error detected" not in r.stdout
+        assert f"turboFFT, {logN}, " in r.stdout

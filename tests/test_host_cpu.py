@@ -1,0 +1,100 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports every
+declared symbol, the host table builders agree with the oracle, the plan CSVs
+are well formed.  No compute call is made (there is no GPU here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import turbofft_amd
+from oracle import turbofft_oracle as O
+from turbofft_amd.codegen import plan as P
+from turbofft_amd.codegen.fft_codegen import KernelSpec, collect_keys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+pytestmark = pytest.mark.skipif(not os.path.exists(turbofft_amd.LIB_PATH),
+                                reason="libturbofft_hip.so not built (python turbofft_amd/build.py)")
+
+
+def test_library_exports_every_declared_symbol():
+    hdr = open(os.path.join(ROOT, "include", "turbofft.h")).read()
+    names = set(re.findall(r"\b(turbofft_[a-z_0-9]+)\s*\(", hdr))
+    assert {"turbofft_plan_create", "turbofft_exec", "turbofft_exec_host", "turbofft_main",
+            "turbofft_get_ft_counters", "turbofft_set_injection"} <= names
+    L = ctypes.CDLL(turbofft_amd.LIB_PATH)
+    for n in sorted(names):
+        assert hasattr(L, n), f"{n} declared in include/turbofft.h but not exported"
+
+
+def test_registry_has_every_kernel_of_the_builtin_plans():
+    have = set(turbofft_amd.kernel_names())
+    for dtype in ("float2", "double2"):
+        rows = P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}.csv"))
+        for key in collect_keys(rows, dtype, [0, 1]):
+            assert key.name in have
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+def test_builtin_rows_match_csv_and_are_consistent(dtype):
+    rows = P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}.csv"))
+    assert len(rows) >= 26
+    for logN in range(1, 26):
+        r = turbofft_amd.builtin_plan_row(dtype, logN)
+        p = P.PlanRow.from_list(r)
+        assert p == rows[logN] and p.logN == logN and sum(p.logNi) == logN
+        for i, k in enumerate(P.kernels_for_row(p, dtype, 0)):
+            sp = KernelSpec(k)
+            assert sp.threads % 64 == 0 and sp.threads <= 1024
+            assert sp.lds_bytes <= 160 * 1024
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        turbofft_amd.builtin_plan_row(dtype, 40)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+def test_twiddle_table_matches_oracle(dtype):
+    a = turbofft_amd.twiddle_table(1 << 12, dtype)
+    b = O.twiddle_table(1 << 12, dtype)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    assert np.max(np.abs(a - b)) <= (1e-7 if dtype == "float2" else 1e-15)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("N", [2, 4, 8, 128, 1024, 8192])
+def test_checksum_vector_exact_matches_oracle(dtype, N):
+    a = turbofft_amd.checksum_vector(N, dtype, "exact")
+    b = O.dft_checksum_vector(N, dtype, "exact")
+    scale = np.max(np.abs(b))
+    assert np.max(np.abs(a - b)) <= scale * (1e-6 if dtype == "float2" else 1e-12)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+def test_checksum_vector_reference_mode_matches_oracle(dtype):
+    # same float-rounded-angle arithmetic on both sides; libm vs numpy sin/cos may
+    # differ in the last ulp of float, so compare to a few ulps of the magnitude
+    N = 256
+    a = turbofft_amd.checksum_vector(N, dtype, "reference")
+    b = O.dft_checksum_vector(N, dtype, "reference")
+    assert np.max(np.abs(a - b)) <= np.max(np.abs(b)) * (2e-5 if dtype == "float2" else 1e-6)
+
+
+def test_bad_arguments_are_reported_not_fatal():
+    L = turbofft_amd.lib()
+    assert L.turbofft_build_twiddle_table(0, 3, None) != 0
+    assert b"power of two" in L.turbofft_last_error()
+    assert L.turbofft_exec(None, None, None, 1, None) != 0
+    # plan creation needs a device: here it must fail with a message, not crash
+    import torch
+    if not torch.cuda.is_available():
+        with pytest.raises(turbofft_amd.TurboFFTError):
+            turbofft_amd.TurboFFT(10, "double2")
+
+
+def test_cli_help_and_bad_flag():
+    import subprocess
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--help"], capture_output=True, text=True)
+    assert r.returncode == 1 and "--if_bench" in r.stdout and "--thread_bs" in r.stdout
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--bogus", "1"], capture_output=True, text=True)
+    assert r.returncode == 1 and "Invalid or incomplete argument: --bogus" in r.stderr

@@ -1,0 +1,224 @@
+"""turbofft_amd -- ctypes binding of libturbofft_hip.so (MI355X / gfx950).
+
+The reference has no Python binding (its test.py only prints dispatch
+tables); this module exposes the C ABI of include/turbofft.h with the
+reference's vocabulary: logN, bs, datatype (0 = float2, 1 = double2), if_ft,
+if_err, thread_bs -- the options of its `turbofft` command line
+(include/utils/CommandLineParser.h:26-45).
+
+There is no CPU fallback: if the HIP library is missing, importing the plan
+class works but creating a plan raises, and every transform runs the
+generated gfx950 kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List, Optional, Tuple
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libturbofft_hip.so")
+CLI_PATH = os.path.join(_HERE, "bin", "turbofft")
+
+FP32, FP64 = 0, 1
+_lib = None
+
+
+class TurboFFTError(RuntimeError):
+    pass
+
+
+def _datatype(dt) -> int:
+    if dt in (0, "float2", "fp32", "f32", np.complex64):
+        return FP32
+    if dt in (1, "double2", "fp64", "f64", np.complex128):
+        return FP64
+    raise ValueError(f"datatype must be 0/float2 or 1/double2, got {dt!r}")
+
+
+def lib() -> C.CDLL:
+    """Load libturbofft_hip.so (built by turbofft_amd/build.py).  Fails loudly."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise TurboFFTError(f"{LIB_PATH} is missing: run `python turbofft_amd/build.py` (there is no CPU fallback)")
+    L = C.CDLL(LIB_PATH)
+    vp, ll, i = C.c_void_p, C.c_longlong, C.c_int
+    L.turbofft_last_error.restype = C.c_char_p
+    L.turbofft_plan_create.restype = vp
+    L.turbofft_plan_create.argtypes = [i, i, i, i, i, C.c_char_p]
+    L.turbofft_plan_destroy.argtypes = [vp]
+    L.turbofft_plan_destroy.restype = None
+    L.turbofft_exec.argtypes = [vp, vp, vp, ll, vp]
+    L.turbofft_exec_host.argtypes = [vp, vp, vp, ll]
+    L.turbofft_time.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_plan_info.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i), C.POINTER(i),
+                                     C.POINTER(C.c_size_t), C.POINTER(i)]
+    L.turbofft_plan_grid.argtypes = [vp, i, ll]
+    L.turbofft_plan_grid.restype = ll
+    L.turbofft_plan_tb_gap.argtypes = [vp, i]
+    L.turbofft_plan_set_tb_gap.argtypes = [vp, i, i]
+    L.turbofft_set_ft_params.argtypes = [vp, C.c_double, C.c_double, i]
+    L.turbofft_set_injection.argtypes = [vp, i, i, i, ll, i, i, C.c_double]
+    L.turbofft_get_ft_counters.argtypes = [vp] + [C.POINTER(C.c_ulonglong)] * 4 + [C.POINTER(ll), i, C.POINTER(i)]
+    L.turbofft_reset_ft_counters.argtypes = [vp]
+    L.turbofft_build_twiddle_table.argtypes = [i, ll, vp]
+    L.turbofft_build_checksum_vector.argtypes = [i, ll, i, vp]
+    L.turbofft_builtin_plan_row.argtypes = [i, i, C.POINTER(i)]
+    L.turbofft_kernel_name.restype = C.c_char_p
+    L.turbofft_kernel_name.argtypes = [i]
+    L.turbofft_main.argtypes = [i, C.POINTER(C.c_char_p)]
+    _lib = L
+    return L
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise TurboFFTError(lib().turbofft_last_error().decode() or f"turbofft error {rc}")
+
+
+# ---- host tables (no GPU needed) ------------------------------------------
+def twiddle_table(N: int, datatype) -> np.ndarray:
+    dt = _datatype(datatype)
+    out = np.empty(2 * N - 1, dtype=np.complex64 if dt == FP32 else np.complex128)
+    _check(lib().turbofft_build_twiddle_table(dt, N, out.ctypes.data))
+    return out
+
+
+def checksum_vector(N: int, datatype, mode: str = "exact") -> np.ndarray:
+    dt = _datatype(datatype)
+    out = np.empty(N, dtype=np.complex64 if dt == FP32 else np.complex128)
+    _check(lib().turbofft_build_checksum_vector(dt, N, {"exact": 0, "reference": 1}[mode], out.ctypes.data))
+    return out
+
+
+def builtin_plan_row(datatype, logN: int) -> List[int]:
+    row = (C.c_int * 11)()
+    _check(lib().turbofft_builtin_plan_row(_datatype(datatype), logN, row))
+    return list(row)
+
+
+def kernel_names() -> List[str]:
+    L = lib()
+    return [L.turbofft_kernel_name(i).decode() for i in range(L.turbofft_kernel_count())]
+
+
+def turbofft_main(argv: List[str]) -> int:
+    """Run the `turbofft` command line in-process."""
+    args = [b"turbofft"] + [a.encode() for a in argv]
+    arr = (C.c_char_p * len(args))(*args)
+    return lib().turbofft_main(len(args), arr)
+
+
+class TurboFFT:
+    """A plan for `bs` forward C2C transforms of length 2^logN."""
+
+    def __init__(self, logN: int, datatype=FP32, if_ft: int = 0, if_err: int = 0, thread_bs: int = 1,
+                 param_csv: Optional[str] = None):
+        self.logN = int(logN)
+        self.N = 1 << self.logN
+        self.datatype = _datatype(datatype)
+        self.cdtype = np.complex64 if self.datatype == FP32 else np.complex128
+        self.if_ft = int(bool(if_ft or if_err))
+        self.if_err = int(bool(if_err))
+        self.thread_bs = int(thread_bs)
+        self._h = lib().turbofft_plan_create(self.logN, self.datatype, self.if_ft, self.if_err, self.thread_bs,
+                                             param_csv.encode() if param_csv else None)
+        if not self._h:
+            raise TurboFFTError(lib().turbofft_last_error().decode())
+        i3 = (C.c_int * 3)
+        n = C.c_int()
+        a, b, c, t = i3(), i3(), i3(), i3()
+        lds = (C.c_size_t * 3)()
+        _check(lib().turbofft_plan_info(self._h, C.byref(n), a, b, c, lds, t))
+        self.launches = n.value
+        self.logNi, self.BS, self.n = list(a)[:n.value], list(b)[:n.value], list(c)[:n.value]
+        self.lds_bytes, self.threads = list(lds)[:n.value], list(t)[:n.value]
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().turbofft_plan_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    # ---- geometry ----
+    def out_elems(self, bs: int) -> int:
+        """Elements the output buffer must hold (workspace included)."""
+        return self.N * bs * (2 if self.launches > 1 else 1)
+
+    def grid(self, launch: int, bs: int) -> int:
+        return lib().turbofft_plan_grid(self._h, launch, bs)
+
+    def tb_gap(self, launch: int) -> int:
+        return lib().turbofft_plan_tb_gap(self._h, launch)
+
+    def set_tb_gap(self, launch: int, gap: int):
+        _check(lib().turbofft_plan_set_tb_gap(self._h, launch, gap))
+
+    # ---- execution ----
+    def exec(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
+        _check(lib().turbofft_exec(self._h, in_ptr, out_ptr, bs, stream))
+
+    def fft(self, x, out=None):
+        """x: torch tensor on the GPU, shape (bs, N), complex64/complex128.
+        Returns a (bs, N) view of the transform (natural order)."""
+        import torch
+        if x.dim() != 2 or x.shape[1] != self.N:
+            raise ValueError(f"expected shape (bs, {self.N}), got {tuple(x.shape)}")
+        want = torch.complex64 if self.datatype == FP32 else torch.complex128
+        if x.dtype != want or not x.is_cuda or not x.is_contiguous():
+            raise ValueError(f"expected a contiguous {want} tensor on the GPU")
+        bs = x.shape[0]
+        if out is None:
+            out = torch.empty(self.out_elems(bs), dtype=want, device=x.device)
+        elif out.numel() < self.out_elems(bs) or out.dtype != want or not out.is_contiguous():
+            raise ValueError(f"out must be contiguous {want} with >= {self.out_elems(bs)} elements")
+        self.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream(x.device).cuda_stream)
+        return out.view(-1)[: bs * self.N].view(bs, self.N)
+
+    def fft_host(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=self.cdtype)
+        if x.ndim != 2 or x.shape[1] != self.N:
+            raise ValueError(f"expected shape (bs, {self.N}), got {x.shape}")
+        out = np.empty_like(x)
+        _check(lib().turbofft_exec_host(self._h, x.ctypes.data, out.ctypes.data, x.shape[0]))
+        return out
+
+    def time(self, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0) -> float:
+        ms = C.c_float()
+        _check(lib().turbofft_time(self._h, in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
+        return ms.value
+
+    # ---- fault tolerance ----
+    def set_ft_params(self, err_smoothing: float = 1000.0, err_threshold: float = 1e-3, correct: bool = True):
+        _check(lib().turbofft_set_ft_params(self._h, err_smoothing, err_threshold, int(correct)))
+
+    def set_injection(self, mode: int, launch: int = -1, every: int = 1, tile_phase: int = 0, s: int = 0, m: int = 0,
+                      mag: float = 100.0):
+        _check(lib().turbofft_set_injection(self._h, mode, launch, every, tile_phase, s, m, mag))
+
+    def reset_ft_counters(self):
+        _check(lib().turbofft_reset_ft_counters(self._h))
+
+    def ft_counters(self, cap: int = 4096) -> dict:
+        v = [C.c_ulonglong() for _ in range(4)]
+        fl = (C.c_longlong * (2 * cap))()
+        n = C.c_int()
+        _check(lib().turbofft_get_ft_counters(self._h, *[C.byref(t) for t in v], fl, cap, C.byref(n)))
+        flagged = [(fl[2 * i], fl[2 * i + 1]) for i in range(n.value)]
+        return {"checked": v[0].value, "detected": v[1].value, "corrected": v[2].value,
+                "uncorrectable": v[3].value, "flagged": flagged}
+
+    # ---- metrics (main.cu:68-69) ----
+    def gflops(self, bs: int, ms: float) -> float:
+        return 5.0 * self.N * self.logN * bs / ms * 1000 / 1e9
+
+    def algorithmic_bytes(self, bs: int) -> int:
+        return 2 * self.N * bs * (8 if self.datatype == FP32 else 16)
+
+    def gbs(self, bs: int, ms: float) -> float:
+        return self.algorithmic_bytes(bs) / ms * 1000 / 1e9

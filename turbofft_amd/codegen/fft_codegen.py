@@ -1,0 +1,720 @@
+#!/usr/bin/env python3
+"""gfx950 kernel generator for the batched radix-2 C2C FFT.
+
+Plays the role of the reference generator
+(include/code_gen/scripts/fft_codegen.py, class TurboFFT + __main__): it reads
+a plan CSV in the reference's 11-column format (logN, launches, logN1..3,
+BS1..3, n1..3; readme.md:48-60) and prints fully unrolled kernels, with the
+same command-line flags (--if_ft, --if_err_injection, --err_smoothing,
+--err_inj, --err_threshold, --datatype, --gpu; fft_codegen.py:709-723).
+
+It is not a translation of that generator.  The differences that matter:
+  * three kernel kinds with run-time geometry -- `row1` (whole transforms,
+    contiguous axis), `col` (strided digit + inter-launch twiddle) and `rowT`
+    (contiguous digit, transposed natural-order store) -- so one kernel per
+    (type, kind, Ni, BS, n) serves every logN with that tile shape;
+  * wave64 thread maps chosen per pass: loads of contiguous rows are
+    row-major (a wavefront reads whole 128-byte lines), the last pass of
+    `rowT` is re-mapped column-major through the final LDS exchange so the
+    transposed store writes BS-element runs;
+  * LDS exchanges with computed padding (see lds_model.py) instead of the
+    rotation swizzle; twiddles W_M^(j*2^b) are fetched exactly from the
+    concatenated table and combined with log-depth products instead of a
+    linear recurrence; inter-launch twiddles use a two-level (hi/lo) table
+    instead of a 2N-entry one;
+  * the fault-tolerance variant keeps the reference's checksum arithmetic
+    (fft_codegen.py:354-384, 432-503) but takes thresholds, the injection
+    descriptor and the correction switch at run time, reports counters, and
+    re-runs the located tile through the same loop body.
+
+Every kernel is emitted as a list of phases separated by block barriers.  The
+same phase text compiles for gfx950 (hipcc) and, with -DTFFT_SIM, as a
+lock-step CPU execution with bounds-checked accessors that the CPU test-suite
+uses to validate index algebra without a GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import math
+import os
+import sys
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+if __package__ in (None, ""):
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
+from turbofft_amd.codegen import lds_model
+from turbofft_amd.codegen.plan import PlanRow, KernelKey, load_plan_csv, kernels_for_row, radix_passes
+
+WAVE = 64
+
+
+def ilog2(v: int) -> int:
+    l = v.bit_length() - 1
+    if v <= 0 or (1 << l) != v:
+        raise ValueError(f"{v} is not a power of two")
+    return l
+
+
+def bitrev(x: int, bits: int) -> int:
+    y = 0
+    for _ in range(bits):
+        y = (y << 1) | (x & 1)
+        x >>= 1
+    return y
+
+
+class Code:
+    def __init__(self):
+        self.lines: List[str] = []
+        self.ind = 0
+
+    def __call__(self, s: str = ""):
+        for ln in s.split("\n"):
+            self.lines.append(("    " * self.ind + ln) if ln else "")
+
+    def text(self) -> str:
+        return "\n".join(self.lines) + "\n"
+
+
+@dataclass
+class KernelSpec:
+    key: KernelKey
+    pad_override: Optional[Dict[int, Tuple[int, int]]] = None
+
+    def __post_init__(self):
+        k = self.key
+        self.T2 = k.dtype                       # float2 / double2
+        self.R = "float" if k.dtype == "float2" else "double"
+        self.esize = 8 if k.dtype == "float2" else 16
+        self.Ni = 1 << k.logNi
+        self.BS = k.BS
+        self.n = k.n
+        self.kind = k.kind
+        self.ft = bool(k.ft)
+        self.passes = radix_passes(self.Ni, self.n)
+        self.npass = len(self.passes)
+        self.Tr = self.Ni // self.n              # threads per sub-FFT
+        self.threads = self.Tr * self.BS
+        self.E = self.Ni * self.BS
+        if self.threads % WAVE or self.threads > 1024:
+            raise ValueError(f"{k}: {self.threads} threads per block (need a multiple of 64, <= 1024)")
+        # thread map per pass: 'major' (s = tx / Tr) or 'minor' (s = tx % BS)
+        if self.kind == "col":
+            self.maps = ["minor"] * self.npass
+        elif self.kind == "row1":
+            self.maps = ["major"] * self.npass
+        else:  # rowT: row-major loads, column-major transposed store
+            self.maps = ["major"] * (self.npass - 1) + ["minor"]
+            if self.npass == 1:
+                self.maps = ["minor"]
+        # P_q: product of the radices before pass q
+        self.P = [1]
+        for R in self.passes:
+            self.P.append(self.P[-1] * R)
+        # padding per exchange x (between pass x and x+1)
+        self.pads: List[Tuple[int, int]] = []
+        for x in range(self.npass - 1):
+            if self.pad_override and x in self.pad_override:
+                self.pads.append(self.pad_override[x])
+            else:
+                self.pads.append(lds_model.choose_padding(self, x))
+        self.lds_elems = max([self.phys_const(self.E - 1, p) + 1 for p in self.pads] + [1])
+        self.red_off_bytes = (self.lds_elems * self.esize + 15) // 16 * 16
+        self.lds_bytes = self.red_off_bytes + (3 * (self.threads // WAVE) * 8 if self.ft else 0)
+
+    # ---- address helpers (python side) ----
+    @staticmethod
+    def phys_const(a: int, pad: Tuple[int, int]) -> int:
+        ps, pl = pad
+        return a if ps < 0 else a + ((a >> ps) << pl)
+
+    def logical_write_addr(self, x: int, tx: int, u: int, o: int) -> int:
+        """Logical LDS element address written by thread tx after pass x for
+        butterfly u, output digit o (layout = thread map of pass x+1)."""
+        s, xr = self.thread_sx(x, tx)
+        R = self.passes[x]
+        P = self.P[x]
+        rest = xr + self.Tr * u
+        low, j = rest % P, rest // P
+        pos = low + P * o + P * R * j
+        return self.layout_addr(self.maps[x + 1], s, pos)
+
+    def logical_read_addr(self, q: int, tx: int, e: int) -> int:
+        s, xr = self.thread_sx(q, tx)
+        return self.layout_addr(self.maps[q], s, xr + self.Tr * e)
+
+    def thread_sx(self, q: int, tx: int) -> Tuple[int, int]:
+        if self.maps[q] == "major":
+            return tx // self.Tr, tx % self.Tr
+        return tx % self.BS, tx // self.BS
+
+    def layout_addr(self, kind: str, s: int, pos: int) -> int:
+        return s * self.Ni + pos if kind == "major" else s + self.BS * pos
+
+    @property
+    def name(self) -> str:
+        return self.key.name
+
+
+class KernelEmitter:
+    def __init__(self, spec: KernelSpec, err_smoothing=1000, err_inj=100, err_threshold=1e-3):
+        self.s = spec
+        self.T2 = spec.T2
+        self.R = spec.R
+
+    # ---------- literals ----------
+    def lit(self, v: float) -> str:
+        if self.R == "float":
+            t = "%.9g" % v
+            if "." not in t and "e" not in t and "n" not in t:
+                t += ".0"
+            return t + "f"
+        t = "%.17g" % v
+        if "." not in t and "e" not in t and "n" not in t:
+            t += ".0"
+        return t
+
+    # ---------- thread map ----------
+    def map_vars(self, c: Code, q: int):
+        sp = self.s
+        if sp.maps[q] == "major":
+            c(f"const unsigned s = tx >> {ilog2(sp.Tr)}, x = tx & {sp.Tr - 1}u;")
+        else:
+            c(f"const unsigned s = tx & {sp.BS - 1}u, x = tx >> {ilog2(sp.BS)};")
+
+    def lds_index(self, expr: str, pad: Tuple[int, int]) -> str:
+        ps, pl = pad
+        if ps < 0:
+            return expr
+        return f"(({expr}) + ((({expr}) >> {ps}) << {pl}))"
+
+    # ---------- radix-R DIF in registers ----------
+    def emit_radix(self, c: Code, regs: Sequence[int]):
+        R = len(regs)
+        length = R
+        while length >= 2:
+            half = length // 2
+            for b0 in range(0, R, length):
+                for k in range(half):
+                    a, b = regs[b0 + k], regs[b0 + k + half]
+                    c(f"t = r[{a}]; r[{a}] = cadd(t, r[{b}]); t = csub(t, r[{b}]);")
+                    # multiply the difference by W_length^k = exp(-2 pi i k/length)
+                    if k == 0:
+                        c(f"r[{b}] = t;")
+                    elif 4 * k == length:
+                        c(f"r[{b}] = cmul_mi(t);")
+                    else:
+                        ang = -2.0 * math.pi * k / length
+                        c(f"r[{b}] = cmulc(t, {self.lit(math.cos(ang))}, {self.lit(math.sin(ang))});")
+            length = half
+
+    # ---------- twiddle powers ----------
+    def emit_apply_powers(self, c: Code, count: int, pow2: Dict[int, str], targets: Sequence[Optional[int]],
+                          base: Optional[str] = None):
+        """Multiply r[targets[e]] by base * w^e for e < count, where pow2[b]
+        names w^(2^b).  Products have depth <= log2(count)."""
+        lo_n = min(count, 8)
+        lo_bits = ilog2(lo_n)
+        wl: Dict[int, Optional[str]] = {0: base}
+        c("{")
+        c.ind += 1
+        for l in range(1, lo_n):
+            hb = l.bit_length() - 1
+            rest = l - (1 << hb)
+            prev = wl[rest]
+            nm = f"wl{l}"
+            if prev is None:
+                c(f"const {self.T2} {nm} = {pow2[hb]};")
+            else:
+                c(f"const {self.T2} {nm} = cmul({prev}, {pow2[hb]});")
+            wl[l] = nm
+        for h in range(count // lo_n):
+            wh = None
+            if h:
+                bits = [b for b in range(8) if (h >> b) & 1]
+                terms = [pow2[lo_bits + b] for b in bits]
+                if len(terms) == 1:
+                    wh = terms[0]
+                else:
+                    c(f"const {self.T2} wh{h} = cmul({terms[0]}, {terms[1]});" if len(terms) == 2 else
+                      f"const {self.T2} wh{h} = cmul(cmul({terms[0]}, {terms[1]}), {terms[2]});")
+                    wh = f"wh{h}"
+            for l in range(lo_n):
+                e = h * lo_n + l
+                tgt = targets[e]
+                if tgt is None:
+                    continue
+                a, b = wl[l], wh
+                if a is None and b is None:
+                    continue
+                if a is None:
+                    w = b
+                elif b is None:
+                    w = a
+                else:
+                    w = f"cmul({a}, {b})"
+                c(f"r[{tgt}] = cmul(r[{tgt}], {w});")
+        c.ind -= 1
+        c("}")
+
+    # ---------- one FFT pass (butterflies + block twiddle) ----------
+    def emit_pass_compute(self, c: Code, q: int):
+        sp = self.s
+        R = sp.passes[q]
+        U = sp.n // R
+        lR = ilog2(R)
+        last = q == sp.npass - 1
+        M = sp.Ni // sp.P[q]
+        c(f"// pass {q}: radix {R}, {U} butterfl{'y' if U == 1 else 'ies'} per thread, sub-FFT length {M}")
+        for u in range(U):
+            self.emit_radix(c, [u + U * i for i in range(R)])
+        if last:
+            return
+        lP = ilog2(sp.P[q])
+        for u in range(U):
+            c("{")
+            c.ind += 1
+            c(f"const unsigned j = (x + {sp.Tr * u}u) >> {lP};")
+            pow2 = {}
+            for b in range(lR):
+                Mb = M >> b
+                c(f"const {self.T2} w{1 << b} = TWLD(tw, {Mb - 1}u + j);   // W_{M}^(j*{1 << b})")
+                pow2[b] = f"w{1 << b}"
+            targets = [u + U * bitrev(o, lR) for o in range(R)]
+            targets[0] = None
+            self.emit_apply_powers(c, R, pow2, targets)
+            c.ind -= 1
+            c("}")
+
+    def emit_lds_write(self, c: Code, q: int):
+        """Store the outputs of pass q in the layout pass q+1 reads."""
+        sp = self.s
+        R = sp.passes[q]
+        U = sp.n // R
+        lR = ilog2(R)
+        P = sp.P[q]
+        lP = ilog2(P)
+        pad = sp.pads[q]
+        nxt = sp.maps[q + 1]
+        for u in range(U):
+            c("{")
+            c.ind += 1
+            c(f"const unsigned rest = x + {sp.Tr * u}u;")
+            c(f"const unsigned pos0 = (rest & {P - 1}u) + ((rest >> {lP}) << {lP + lR});")
+            if nxt == "major":
+                c(f"const unsigned a0 = (s << {ilog2(sp.Ni)}) + pos0;")
+                step = P
+            else:
+                c(f"const unsigned a0 = s + (pos0 << {ilog2(sp.BS)});")
+                step = P * sp.BS
+            for o in range(R):
+                reg = u + U * bitrev(o, lR)
+                c(f"LST({self.lds_index(f'a0 + {step * o}u', pad)}, r[{reg}]);")
+            c.ind -= 1
+            c("}")
+
+    def emit_lds_read(self, c: Code, q: int):
+        sp = self.s
+        pad = sp.pads[q - 1]
+        if sp.maps[q] == "major":
+            c(f"const unsigned b0 = (s << {ilog2(sp.Ni)}) + x;")
+            step = sp.Tr
+        else:
+            c("const unsigned b0 = tx;")
+            step = sp.threads
+        for e in range(sp.n):
+            c(f"r[{e}] = LLD({self.lds_index(f'b0 + {step * e}u', pad)});")
+
+    # ---------- global addressing ----------
+    def emit_tile_decode(self, c: Code):
+        sp = self.s
+        lBS = ilog2(sp.BS)
+        if sp.kind == "row1":
+            c(f"const long long row0 = tile << {lBS};")
+        elif sp.kind == "col":
+            c(f"const unsigned tpl = (unsigned)a.log_ncols - {lBS}u;")
+            c("const unsigned ct = (unsigned)(tile & ((1ll << tpl) - 1));")
+            c("const long long outer = tile >> tpl;")
+            c(f"const long long tbase = (outer << ({ilog2(sp.Ni)} + a.log_ncols)) + ((long long)ct << {lBS});")
+        else:
+            c(f"const unsigned ctl = (unsigned)a.logC - {lBS}u;")
+            c("const unsigned ct = (unsigned)(tile & ((1ll << ctl) - 1));")
+            c("const unsigned qd = (unsigned)((tile >> ctl) & ((1ll << a.logQ) - 1));")
+            c("const long long tb = (tile >> (ctl + a.logQ)) << a.logN;")
+
+    def emit_load(self, c: Code):
+        sp = self.s
+        lNi = ilog2(sp.Ni)
+        if sp.kind == "row1":
+            c(f"const long long gi = ((row0 + s) << {lNi}) + x;")
+            c("const bool ok = (row0 + s) < a.nrows;")
+            for e in range(sp.n):
+                c(f"r[{e}] = ok ? GLD(in, gi + {sp.Tr * e}) : czero(r[0]);")
+        elif sp.kind == "col":
+            c(f"const long long gi = tbase + s + ((long long)x << a.log_ncols);")
+            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
+            for e in range(sp.n):
+                c(f"r[{e}] = GLD(in, gi + {e} * gstep);")
+        else:
+            c(f"const long long gi = tb + ((long long)(qd + (((ct << {ilog2(sp.BS)}) + s) << a.logQ)) << {lNi}) + x;")
+            for e in range(sp.n):
+                c(f"r[{e}] = GLD(in, gi + {sp.Tr * e});")
+
+    def out_reg(self, e: int) -> int:
+        """Register that holds output k = x + Tr*e after the last pass."""
+        sp = self.s
+        R = sp.passes[-1]
+        U = sp.n // R
+        u, o = e % U, e // U
+        return u + U * bitrev(o, ilog2(R))
+
+    def emit_store(self, c: Code):
+        sp = self.s
+        lNi = ilog2(sp.Ni)
+        if sp.kind == "row1":
+            c(f"const long long go = ((row0 + s) << {lNi}) + x;")
+            c("if ((row0 + s) < a.nrows) {")
+            c.ind += 1
+            for e in range(sp.n):
+                c(f"GST(out, go + {sp.Tr * e}, r[{self.out_reg(e)}]);")
+            c.ind -= 1
+            c("}")
+        elif sp.kind == "col":
+            c("const unsigned col = (ct << %d) + s;" % ilog2(sp.BS))
+            self.emit_interlaunch_twiddle(c)
+            c(f"const long long go = tbase + s + ((long long)x << a.log_ncols);")
+            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
+            for e in range(sp.n):
+                c(f"GST(out, go + {e} * gstep, r[{self.out_reg(e)}]);")
+        else:
+            c(f"const unsigned ls = (unsigned)a.logN - {lNi}u;")
+            c(f"const long long go = tb + ((ct << {ilog2(sp.BS)}) + s) + ((long long)qd << a.logC) + ((long long)x << ls);")
+            c(f"const long long gstep = {sp.Tr}ll << ls;")
+            for e in range(sp.n):
+                c(f"GST(out, go + {e} * gstep, r[{self.out_reg(e)}]);")
+
+    def emit_interlaunch_twiddle(self, c: Code):
+        """r[k] *= W_(Ni*ncols)^(col*k), k = x + Tr*e: base and step come from the
+        two-level table, powers of the step by squaring."""
+        sp = self.s
+        n = sp.n
+        c("{")
+        c.ind += 1
+        c(f"const unsigned L = {ilog2(sp.Ni)}u + (unsigned)a.log_ncols;")
+        c("const unsigned emask = (L >= 32u) ? 0xffffffffu : ((1u << L) - 1u);")
+        c("const unsigned lomask = (1u << a.tw_lo_bits) - 1u;")
+        c("const unsigned e0 = (col * x) & emask;")
+        c(f"const unsigned e1 = (col * {sp.Tr}u) & emask;")
+        c(f"const {self.T2} wb = cmul(TWLD(twhi, e0 >> a.tw_lo_bits), TWLD(twlo, e0 & lomask));")
+        pow2 = {}
+        if n > 1:
+            c(f"const {self.T2} d1 = cmul(TWLD(twhi, e1 >> a.tw_lo_bits), TWLD(twlo, e1 & lomask));")
+            pow2[0] = "d1"
+            for b in range(1, ilog2(n)):
+                c(f"const {self.T2} d{1 << b} = cmul(d{1 << (b - 1)}, d{1 << (b - 1)});")
+                pow2[b] = f"d{1 << b}"
+        targets = [self.out_reg(e) for e in range(n)]
+        self.emit_apply_powers(c, n, pow2, targets, base="wb")
+        c.ind -= 1
+        c("}")
+
+    # ---------- fault tolerance ----------
+    def emit_ft_input(self, c: Code):
+        """in1 += re+im of x*c[m]; in2 += cnt * (...)   (fft_codegen.py:354-367),
+        then the optional compute-side error injection (:412-415)."""
+        sp = self.s
+        c("if (!is_redo) {")
+        c.ind += 1
+        c(f"{self.R} acc = 0;")
+        for e in range(sp.n):
+            c(f"{{ const {self.T2} cv = TWLD(ck, x + {sp.Tr * e}u); const {self.T2} p = cmul(r[{e}], cv); acc += p.x + p.y; }}")
+        c("fin1 += acc; fin2 += cntf * acc;")
+        c("if (inj_hit && s == (unsigned)a.ft.inj_s && x == ((unsigned)a.ft.inj_m & %du)) {" % (sp.Tr - 1))
+        c.ind += 1
+        c(f"const unsigned ie = (unsigned)a.ft.inj_m >> {ilog2(sp.Tr)};")
+        for e in range(sp.n):
+            c(f"if (ie == {e}u) r[{e}].x += ({self.R})a.ft.inj_mag;")
+        c.ind -= 1
+        c("}")
+        c.ind -= 1
+        c("}")
+
+    def emit_ft_output(self, c: Code):
+        """out1 -= re+im of y*r[k%3]; out2 -= cnt * (...)   (fft_codegen.py:374-384),
+        taken before the inter-launch twiddle."""
+        sp = self.s
+        c("if (!is_redo) {")
+        c.ind += 1
+        c("const unsigned x3 = x % 3u;")
+        s3 = self.lit(0.8660253882408142)
+        c(f"const {self.R} rrx0 = (x3 == 0u) ? ({self.R})1 : ({self.R})-0.5;")
+        c(f"const {self.R} rry0 = (x3 == 0u) ? ({self.R})0 : ((x3 == 1u) ? -{s3} : {s3});")
+        c(f"const {self.R} rrx1 = (x3 == 2u) ? ({self.R})1 : ({self.R})-0.5;")
+        c(f"const {self.R} rry1 = (x3 == 2u) ? ({self.R})0 : ((x3 == 0u) ? -{s3} : {s3});")
+        c(f"const {self.R} rrx2 = (x3 == 1u) ? ({self.R})1 : ({self.R})-0.5;")
+        c(f"const {self.R} rry2 = (x3 == 1u) ? ({self.R})0 : ((x3 == 2u) ? -{s3} : {s3});")
+        c(f"{self.R} acc = 0;")
+        for e in range(sp.n):
+            ce = (sp.Tr * e) % 3
+            reg = self.out_reg(e)
+            c(f"{{ const {self.T2} p = cmulc(r[{reg}], rrx{ce}, rry{ce}); acc += p.x + p.y; }}")
+        c("fo1 -= acc; fo2 -= cntf * acc;")
+        c.ind -= 1
+        c("}")
+
+    # ---------- phases ----------
+    def phases(self) -> List[str]:
+        sp = self.s
+        out: List[str] = []
+        for q in range(sp.npass):
+            c = Code()
+            self.map_vars(c, q)
+            c(f"{self.T2} t;")
+            if q == 0:
+                self.emit_load(c)
+                if sp.ft:
+                    self.emit_ft_input(c)
+            else:
+                self.emit_lds_read(c, q)
+            self.emit_pass_compute(c, q)
+            if q == sp.npass - 1:
+                if sp.ft:
+                    self.emit_ft_output(c)
+                self.emit_store(c)
+                c("(void)t;")
+                out.append(c.text())
+            else:
+                c("(void)t;")
+                out.append(c.text())
+                w = Code()
+                self.map_vars(w, q)
+                self.emit_lds_write(w, q)
+                out.append(w.text())
+        return out
+
+    # ---------- whole kernel ----------
+    def emit(self, sim: bool) -> str:
+        sp = self.s
+        c = Code()
+        T2, R = self.T2, self.R
+        c(f"// {sp.name}: {sp.kind} kernel, {T2}, Ni={sp.Ni}, BS={sp.BS}, n={sp.n}, passes={'x'.join(map(str, sp.passes))},")
+        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
+        if sim:
+            c(f'extern "C" void {sp.name}_sim(const {T2}* in, {T2}* out, const {T2}* tw, const tfft_kargs* ap, long long grid, const long long* limits)')
+            c("{")
+            c.ind += 1
+            c("const tfft_kargs a = *ap;")
+            c("const long long in_limit = limits[0], out_limit = limits[1], tw_limit = limits[2];")
+            c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
+            c(f"const long long lds_limit = {sp.lds_elems};")
+            c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c("for (long long bx = 0; bx < grid; ++bx) {")
+            c.ind += 1
+            c(f"std::vector<{T2}> ldsv({sp.lds_elems}); {T2}* lds = ldsv.data();")
+            c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
+        else:
+            c(f'extern "C" __global__ __launch_bounds__({sp.threads})')
+            c(f"void {sp.name}(const {T2}* __restrict__ in, {T2}* __restrict__ out, const {T2}* __restrict__ tw, const tfft_kargs a)")
+            c("{")
+            c.ind += 1
+            c("extern __shared__ __align__(16) unsigned char lds_raw[];")
+            c(f"{T2}* lds = ({T2}*)lds_raw;")
+            c("const unsigned tx = threadIdx.x;")
+            c("const long long bx = blockIdx.x, grid = gridDim.x;")
+            c(f"{T2} r[{sp.n}];")
+            if sp.ft:
+                c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
+        c(f"const {T2}* twhi = (const {T2}*)a.tw_hi; const {T2}* twlo = (const {T2}*)a.tw_lo; const {T2}* ck = (const {T2}*)a.ft.cksum;")
+        c("(void)twhi; (void)twlo; (void)ck;")
+        # tile group of this block (fft_codegen.py:218,260-261 with a rounded-up grid)
+        c("const long long chunk = bx / a.tb_gap;")
+        c("const long long gstride = ((chunk + 1) * a.tb_gap <= grid) ? a.tb_gap : (grid - chunk * a.tb_gap);")
+        c("const long long tile0 = chunk * a.tb_gap * a.thread_bs + bx % a.tb_gap;")
+        c("int count = 0;")
+        c("if (tile0 < a.ntiles) { const long long left = (a.ntiles - tile0 + gstride - 1) / gstride; count = left < a.thread_bs ? (int)left : a.thread_bs; }")
+        if sp.ft:
+            c("long long redo_tile = -1; int extra = 0;")
+            c("for (int it = 0; it < count + extra; ++it) {")
+            c.ind += 1
+            c("const bool is_redo = it >= count;")
+            c("const long long tile = is_redo ? redo_tile : tile0 + it * gstride;")
+            c(f"const {R} cntf = ({R})(it + 1);")
+            c("bool inj_hit = false;")
+            c("if (a.ft.inj_mode == 1) inj_hit = (it == (int)(bx % a.thread_bs)) && (bx % a.ft.inj_every == 0);")
+            c("else if (a.ft.inj_mode == 2) inj_hit = (tile % a.ft.inj_every) == a.ft.inj_tile;")
+            c("(void)cntf; (void)inj_hit;")
+        else:
+            c("for (int it = 0; it < count; ++it) {")
+            c.ind += 1
+            c("const long long tile = tile0 + it * gstride;")
+        self.emit_tile_decode(c)
+        phases = self.phases()
+        for i, ph in enumerate(phases):
+            if i:
+                if sim:
+                    c("// ---- barrier ----")
+                else:
+                    c("__syncthreads();")
+            if sim:
+                c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
+                c.ind += 1
+                c("auto& r = ts[tx].r; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
+                c("(void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+            else:
+                c("{")
+                c.ind += 1
+            c(ph.rstrip("\n"))
+            c.ind -= 1
+            c("}")
+        if sp.ft:
+            self.emit_ft_decide(c, sim)
+        c.ind -= 1
+        c("}")  # tile loop
+        if sim:
+            c.ind -= 1
+            c("}")  # block loop
+        c.ind -= 1
+        c("}")
+        return c.text()
+
+    def emit_ft_decide(self, c: Code, sim: bool):
+        """Block-wide reduction and the detect / locate decision
+        (fft_codegen.py:432-503), then scheduling of the recompute."""
+        sp = self.s
+        R = self.R
+        nw = sp.threads // WAVE
+        c("if (it == count - 1) {")
+        c.ind += 1
+        c(f"{R} delta, mag, delta2;")
+        if sim:
+            c("delta = 0; mag = 0; delta2 = 0;")
+            c("for (auto& z : ts) { delta += z.fin1 + z.fo1; mag += fabs(z.fo1) + fabs(z.fin1); delta2 += z.fin2 + z.fo2; }")
+            c("const unsigned tx = 0;")
+        else:
+            c(f"{R}* red = ({R}*)(lds_raw + {sp.red_off_bytes});")
+            c(f"{R} v0 = wave_sum(fin1 + fo1), v1 = wave_sum(fabs(fo1) + fabs(fin1)), v2 = wave_sum(fin2 + fo2);")
+            c("if ((tx & 63u) == 0u) { red[(tx >> 6) * 3 + 0] = v0; red[(tx >> 6) * 3 + 1] = v1; red[(tx >> 6) * 3 + 2] = v2; }")
+            c("__syncthreads();")
+            c("delta = 0; mag = 0; delta2 = 0;")
+            c(f"for (int w = 0; w < {nw}; ++w) {{ delta += red[w * 3 + 0]; mag += red[w * 3 + 1]; delta2 += red[w * 3 + 2]; }}")
+        c(f"const bool det = fabs(delta) / (({R})a.ft.err_smoothing + fabs(mag)) > ({R})a.ft.err_threshold;")
+        c("int k = -1;")
+        c("if (det) k = (int)round(fabs(delta2) / fabs(delta));")
+        c("const bool valid = det && k >= 1 && k <= count;")
+        c("const long long bad = valid ? tile0 + (long long)(k - 1) * gstride : -1;")
+        c("if (tx == 0) {")
+        c.ind += 1
+        if sim:
+            c("a.ft.counters[0] += 1;")
+            c("if (det) {")
+            c("    a.ft.counters[1] += 1;")
+            c("    const unsigned long long slot = a.ft.counters[4]++;")
+            c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
+            c("    if (valid && a.ft.correct) a.ft.counters[2] += 1;")
+            c("    if (!valid) a.ft.counters[3] += 1;")
+            c("}")
+        else:
+            c("atomicAdd(&a.ft.counters[0], 1ull);")
+            c("if (det) {")
+            c("    atomicAdd(&a.ft.counters[1], 1ull);")
+            c("    const unsigned long long slot = atomicAdd(&a.ft.counters[4], 1ull);")
+            c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
+            c("    if (valid && a.ft.correct) atomicAdd(&a.ft.counters[2], 1ull);")
+            c("    if (!valid) atomicAdd(&a.ft.counters[3], 1ull);")
+            c("}")
+        c.ind -= 1
+        c("}")
+        c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")
+        c.ind -= 1
+        c("}")
+
+
+FILE_HEADER = """// GENERATED by turbofft_amd/codegen/fft_codegen.py -- do not edit.
+#include "../tfft_device.h"
+"""
+
+
+def generate_source(specs: Sequence[KernelSpec], sim: bool) -> str:
+    out = [FILE_HEADER]
+    if sim:
+        out[0] = FILE_HEADER.replace('#include "../tfft_device.h"', '#define TFFT_SIM 1\n#include "../tfft_device.h"')
+    for sp in specs:
+        out.append(KernelEmitter(sp).emit(sim))
+    return "\n".join(out)
+
+
+def registry_source(specs: Sequence[KernelSpec]) -> str:
+    """C table the host driver uses to find a kernel for a launch
+    (the role of TurboFFT_Kernel_Entry, include/TurboFFT.h:22-25,118-526)."""
+    c = Code()
+    c("// GENERATED by turbofft_amd/codegen/fft_codegen.py -- do not edit.")
+    c('#include <hip/hip_runtime.h>')
+    c('#include "../tfft_registry.h"')
+    for sp in specs:
+        c(f'extern "C" __global__ void {sp.name}(const {sp.T2}*, {sp.T2}*, const {sp.T2}*, const tfft_kargs);')
+    c("static const tfft_kernel_entry tfft_kernel_table_[] = {")
+    kinds = {"row1": 0, "col": 1, "rowT": 2}
+    for sp in specs:
+        k = sp.key
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {sp.threads}, {sp.lds_bytes}}},')
+    c("};")
+    c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
+    c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")
+    c("    return tfft_kernel_table_;")
+    c("}")
+    return c.text()
+
+
+def collect_keys(rows: Sequence[PlanRow], dtype: str, ft_variants: Sequence[int]) -> List[KernelKey]:
+    keys: List[KernelKey] = []
+    seen = set()
+    for row in rows:
+        if row.launches == 0:
+            continue
+        for ft in ft_variants:
+            for k in kernels_for_row(row, dtype, ft):
+                if k not in seen:
+                    seen.add(k)
+                    keys.append(k)
+    return keys
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="turboFFT gfx950 kernel generator.")
+    # the reference generator's flags (fft_codegen.py:709-723)
+    ap.add_argument("--if_ft", type=int, default=0, help="emit the fault-tolerant variants (0/1)")
+    ap.add_argument("--if_err_injection", type=int, default=0,
+                    help="accepted for compatibility: injection and correction are run-time switches of the FT kernels")
+    ap.add_argument("--err_smoothing", type=int, default=1000, help="default only; passed at run time")
+    ap.add_argument("--err_inj", type=int, default=100, help="default only; passed at run time")
+    ap.add_argument("--err_threshold", type=float, default=1e-3, help="default only; passed at run time")
+    ap.add_argument("--datatype", type=str, default="double2")
+    ap.add_argument("--gpu", type=str, default="gfx950")
+    # this generator's own
+    ap.add_argument("--param", type=str, default=None, help="plan CSV (default: param/<gpu>/param_<datatype>.csv)")
+    ap.add_argument("--outdir", type=str, default=None)
+    ap.add_argument("--sim", type=int, default=0, help="emit the CPU lock-step flavour")
+    ap.add_argument("--list", action="store_true", help="print the kernel names and exit")
+    args = ap.parse_args(argv)
+    here = os.path.dirname(os.path.abspath(__file__))
+    param = args.param or os.path.join(here, "..", "param", args.gpu, f"param_{args.datatype}.csv")
+    rows = load_plan_csv(param)
+    keys = collect_keys(rows, args.datatype, [1] if args.if_ft else [0])
+    specs = [KernelSpec(k) for k in keys]
+    if args.list:
+        for sp in specs:
+            print(sp.name, sp.threads, sp.lds_bytes, sp.passes, sp.pads)
+        return 0
+    outdir = args.outdir or os.path.join(here, "..", "csrc", "generated")
+    os.makedirs(outdir, exist_ok=True)
+    for sp in specs:
+        path = os.path.join(outdir, sp.name + (".sim.cpp" if args.sim else ".hip"))
+        with open(path, "w") as f:
+            f.write(generate_source([sp], bool(args.sim)))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,78 @@
+"""LDS bank-conflict model used to pick the padding of every exchange.
+
+gfx950 LDS is modelled as 64 banks of 4 bytes.  An access of `esize` bytes per
+lane is served in groups of (256 / esize) lanes per cycle; a group costs as
+many cycles as the worst bank is hit by distinct addresses.  Reads are
+unit-stride across lanes by construction (the layout of an exchange follows
+the thread map of the pass that reads it), so only the writes are scored.
+
+Padding is phys(a) = a + ((a >> ps) << pl) in elements; (-1, 0) means none.
+"""
+from __future__ import annotations
+
+from typing import List, Tuple
+
+BANKS = 64
+BANK_BYTES = 4
+
+
+def access_cost(byte_addrs: List[int], esize: int) -> int:
+    lanes_per_group = max(1, (BANKS * BANK_BYTES) // esize)
+    cost = 0
+    for g in range(0, len(byte_addrs), lanes_per_group):
+        per_bank = {}
+        for a in byte_addrs[g:g + lanes_per_group]:
+            for w in range(esize // BANK_BYTES):
+                b = ((a // BANK_BYTES) + w) % BANKS
+                per_bank.setdefault(b, set()).add(a // BANK_BYTES + w)
+        cost += max(len(v) for v in per_bank.values())
+    return cost
+
+
+def exchange_write_cost(spec, x: int, pad: Tuple[int, int]) -> Tuple[int, int]:
+    """(cycles, ideal cycles) for wavefront 0 writing the outputs of pass x."""
+    R = spec.passes[x]
+    U = spec.n // R
+    total = 0
+    ideal = 0
+    waves = [0] if spec.threads <= 64 else [0, spec.threads // 64 - 1]
+    for w in waves:
+        for u in range(U):
+            for o in range(R):
+                addrs = [spec.phys_const(spec.logical_write_addr(x, w * 64 + lane, u, o), pad) * spec.esize
+                         for lane in range(64)]
+                total += access_cost(addrs, spec.esize)
+                ideal += max(1, 64 * spec.esize // (BANKS * BANK_BYTES))
+    return total, ideal
+
+
+def exchange_read_cost(spec, x: int, pad: Tuple[int, int]) -> Tuple[int, int]:
+    total = 0
+    ideal = 0
+    for e in range(spec.n):
+        addrs = [spec.phys_const(spec.logical_read_addr(x + 1, lane, e), pad) * spec.esize for lane in range(64)]
+        total += access_cost(addrs, spec.esize)
+        ideal += max(1, 64 * spec.esize // (BANKS * BANK_BYTES))
+    return total, ideal
+
+
+def choose_padding(spec, x: int) -> Tuple[int, int]:
+    """Smallest-cost (ps, pl) for exchange x; ties go to the least extra LDS."""
+    E = spec.E
+    best = None
+    cands = [(-1, 0)]
+    for ps in range(1, max(2, E.bit_length() - 1)):
+        for pl in range(0, 5):
+            if (1 << pl) >= (1 << ps):
+                continue
+            cands.append((ps, pl))
+    for pad in cands:
+        w, _ = exchange_write_cost(spec, x, pad)
+        r, _ = exchange_read_cost(spec, x, pad)
+        extra = spec.phys_const(E - 1, pad) + 1 - E
+        if extra * 8 > E:          # at most 12.5 % extra LDS
+            continue
+        score = (w + r, extra)
+        if best is None or score < best[0]:
+            best = (score, pad)
+    return best[1]

@@ -1,0 +1,88 @@
+"""Plan rows and the kernels they need.
+
+A plan CSV keeps the reference's 11-column row
+`logN, launches, logN1, logN2, logN3, BS1, BS2, BS3, n1, n2, n3`
+(readme.md:48-60; consumed at fft_codegen.py:745-752 and main.cu:8-9,16,22-24),
+row index == logN.  Launch i transforms a digit of size 2^logNi with BSi
+sub-FFTs per tile and ni elements per thread; launch 0 owns the most-strided
+digit and the last launch the contiguous one.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Sequence, Tuple
+
+
+@dataclass(frozen=True)
+class PlanRow:
+    logN: int
+    launches: int
+    logNi: Tuple[int, ...]
+    BS: Tuple[int, ...]
+    n: Tuple[int, ...]
+
+    @staticmethod
+    def from_list(row: Sequence[int]) -> "PlanRow":
+        row = [int(v) for v in row]
+        if len(row) < 11:
+            raise ValueError(f"plan row needs 11 columns, got {len(row)}: {row}")
+        L = row[1]
+        if not 0 <= L <= 3:
+            raise ValueError(f"launches must be 0..3: {row}")
+        p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]))
+        if L and sum(p.logNi) != p.logN:
+            raise ValueError(f"logN1+logN2+logN3 != logN in row {row}")
+        return p
+
+    @property
+    def N(self) -> int:
+        return 1 << self.logN
+
+
+@dataclass(frozen=True)
+class KernelKey:
+    dtype: str       # "float2" | "double2"
+    kind: str        # "row1" | "col" | "rowT"
+    logNi: int
+    BS: int
+    n: int
+    ft: int
+
+    @property
+    def name(self) -> str:
+        t = "f32" if self.dtype == "float2" else "f64"
+        return f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_ft" if self.ft else "")
+
+
+def load_plan_csv(path: str) -> List[PlanRow]:
+    rows = []
+    with open(path) as f:
+        for line in f:
+            line = line.strip()
+            if not line or line.startswith("#"):
+                continue
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:11]]))
+    return rows
+
+
+def launch_kinds(launches: int) -> List[str]:
+    return {1: ["row1"], 2: ["col", "rowT"], 3: ["col", "col", "rowT"]}[launches]
+
+
+def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
+    return [KernelKey(dtype, kind, row.logNi[i], row.BS[i], row.n[i], int(ft))
+            for i, kind in enumerate(launch_kinds(row.launches))]
+
+
+def radix_passes(Ni: int, n: int) -> List[int]:
+    """Pass radices inside a block: n, n, ..., leftover (leftover last), the
+    same split the reference uses (fft_codegen.py:36-43, 127-138)."""
+    if n > Ni:
+        raise ValueError(f"n={n} exceeds the sub-FFT length {Ni}")
+    out = []
+    m = Ni
+    while m > 1:
+        r = n if m >= n else m
+        out.append(r)
+        m //= r
+    return out

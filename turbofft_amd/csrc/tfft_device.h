@@ -1,0 +1,84 @@
+// Device-side helpers shared by every generated kernel.
+//
+// The generated code is written once and compiled two ways:
+//   * hipcc --offload-arch=gfx950          -> the product kernels;
+//   * g++ -DTFFT_SIM (tests only)          -> a lock-step CPU execution of the
+//     same phase list with bounds-checked global / LDS accessors, used to
+//     catch index and barrier-placement mistakes without a GPU.
+// Complex arithmetic mirrors the reference's 2-op add/sub and 4-op multiply
+// (include/turbofft/macro_ops.h:14-18).
+#pragma once
+#include "../../include/turbofft_kargs.h"
+
+#ifndef TFFT_SIM
+#include <hip/hip_runtime.h>
+#define TFFT_DEV __device__ __forceinline__
+#define GLD(p, i) ((p)[(i)])
+#define GST(p, i, v) ((p)[(i)] = (v))
+#define TWLD(p, i) ((p)[(i)])
+#define LLD(i) (lds[(i)])
+#define LST(i, v) (lds[(i)] = (v))
+#else
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+struct float2 { float x, y; };
+struct double2 { double x, y; };
+#define TFFT_DEV static inline
+struct tfft_sim_bounds_t { long long in_elems, out_elems, tw_elems, lds_elems, twhi_elems, twlo_elems; };
+extern tfft_sim_bounds_t tfft_sim_bounds;
+extern long long tfft_sim_errors;
+#define TFFT_CHK(i, n, what)                                                              \
+    (((long long)(i) < 0 || (long long)(i) >= (long long)(n))                             \
+         ? (tfft_sim_errors++ == 0 ? fprintf(stderr, "tfft sim: %s index %lld out of [0,%lld) at %s:%d\n", \
+                                             what, (long long)(i), (long long)(n), __FILE__, __LINE__) : 0, 0LL) \
+         : (long long)(i))
+#define GLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
+#define GST(p, i, v) ((p)[TFFT_CHK((i), p##_limit, #p)] = (v))
+#define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
+#define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
+#define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
+#endif
+
+TFFT_DEV float2 cadd(float2 a, float2 b) { float2 c; c.x = a.x + b.x; c.y = a.y + b.y; return c; }
+TFFT_DEV float2 csub(float2 a, float2 b) { float2 c; c.x = a.x - b.x; c.y = a.y - b.y; return c; }
+TFFT_DEV float2 cmul(float2 a, float2 b) { float2 c; c.x = a.x * b.x - a.y * b.y; c.y = a.y * b.x + a.x * b.y; return c; }
+TFFT_DEV float2 cmulc(float2 a, float cr, float ci) { float2 c; c.x = a.x * cr - a.y * ci; c.y = a.y * cr + a.x * ci; return c; }
+TFFT_DEV float2 cmul_mi(float2 a) { float2 c; c.x = a.y; c.y = -a.x; return c; }   // * (-i)
+TFFT_DEV float2 cmul_pi(float2 a) { float2 c; c.x = -a.y; c.y = a.x; return c; }   // * (+i)
+TFFT_DEV float2 cneg(float2 a) { float2 c; c.x = -a.x; c.y = -a.y; return c; }
+TFFT_DEV float2 czero(float2) { float2 c; c.x = 0.f; c.y = 0.f; return c; }
+
+TFFT_DEV double2 cadd(double2 a, double2 b) { double2 c; c.x = a.x + b.x; c.y = a.y + b.y; return c; }
+TFFT_DEV double2 csub(double2 a, double2 b) { double2 c; c.x = a.x - b.x; c.y = a.y - b.y; return c; }
+TFFT_DEV double2 cmul(double2 a, double2 b) { double2 c; c.x = a.x * b.x - a.y * b.y; c.y = a.y * b.x + a.x * b.y; return c; }
+TFFT_DEV double2 cmulc(double2 a, double cr, double ci) { double2 c; c.x = a.x * cr - a.y * ci; c.y = a.y * cr + a.x * ci; return c; }
+TFFT_DEV double2 cmul_mi(double2 a) { double2 c; c.x = a.y; c.y = -a.x; return c; }
+TFFT_DEV double2 cmul_pi(double2 a) { double2 c; c.x = -a.y; c.y = a.x; return c; }
+TFFT_DEV double2 cneg(double2 a) { double2 c; c.x = -a.x; c.y = -a.y; return c; }
+TFFT_DEV double2 czero(double2) { double2 c; c.x = 0.0; c.y = 0.0; return c; }
+
+#ifndef TFFT_SIM
+// Sum over the 64 lanes of a wavefront; every lane receives the total.
+// Steps 1 and 2 are DPP quad permutes, 4/8/16 go through the ds_swizzle
+// crossbar (no LDS memory is touched), 32 uses a permute across the two halves.
+TFFT_DEV float wave_sum(float v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+TFFT_DEV double wave_sum(double v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+#endif

@@ -1,0 +1,21 @@
+// Kernel registry entry emitted by the generator: the role of the reference's
+// TurboFFT_Kernel_Entry<T, ft, err, arch>::turboFFTArr[logN][launch] function
+// pointer table (include/TurboFFT.h:22-25, 118-526), keyed by tile shape
+// instead of by logN.
+#pragma once
+#include "../../include/turbofft_kargs.h"
+
+typedef struct tfft_kernel_entry {
+    const char* name;
+    const void* func;    // host-side kernel handle for hipLaunchKernel
+    int datatype;        // 0 = float2, 1 = double2
+    int kind;            // 0 = row1, 1 = col, 2 = rowT
+    int logNi, BS, n, ft;
+    int threads;         // block size
+    int lds_bytes;       // dynamic LDS
+} tfft_kernel_entry;
+
+#ifdef __cplusplus
+extern "C"
+#endif
+const tfft_kernel_entry* tfft_kernel_table(int* count);

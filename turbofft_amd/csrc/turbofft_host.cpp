@@ -1,0 +1,588 @@
+// Host driver behind the C ABI in include/turbofft.h.
+//
+// Mirrors the host side of the reference (main.cu:4-73 test_turbofft,
+// include/utils/initializeData.h, include/utils/abft.h, include/utils/readCSV.h)
+// for MI355X: plan rows come from the reference's 11-column CSV format, kernels
+// from the generated registry, geometry is passed to the kernels at launch.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/turbofft.h"
+#include "tfft_registry.h"
+
+extern "C" const char* tfft_builtin_param_csv(int datatype);   // generated: the gfx950 CSV text
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                         \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess)                                                                 \
+            return fail(TURBOFFT_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                        __FILE__, __LINE__);                                                  \
+    } while (0)
+
+constexpr double kPi = 3.14159265358979323846;
+constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
+
+struct Row {
+    int v[11];
+    int logN() const { return v[0]; }
+    int launches() const { return v[1]; }
+    int logNi(int i) const { return v[2 + i]; }
+    int BS(int i) const { return v[5 + i]; }
+    int n(int i) const { return v[8 + i]; }
+};
+
+// readCSV.h:3-33: split on ',' and atoi; row index == logN.
+bool parse_csv(std::istream& in, std::vector<Row>& rows) {
+    std::string line;
+    while (std::getline(in, line)) {
+        if (line.find_first_not_of(" \t\r\n") == std::string::npos) continue;
+        if (line[line.find_first_not_of(" \t")] == '#') continue;
+        Row r;
+        memset(&r, 0, sizeof r);
+        std::istringstream ls(line);
+        std::string tok;
+        int c = 0;
+        while (c < 11 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        if (c < 11) return false;
+        rows.push_back(r);
+    }
+    return true;
+}
+
+int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
+    if (launches == 1) return 0;
+    return i == launches - 1 ? 2 : 1;
+}
+
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft) {
+    int cnt = 0;
+    const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
+    for (int i = 0; i < cnt; ++i)
+        if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
+            t[i].n == n && t[i].ft == ft)
+            return &t[i];
+    return nullptr;
+}
+
+template <class C>
+void fill_twiddle(C* out, long long N) {
+    // initializeData.h:31-37: for c = 1,2,4..N, tw[c-1+m] = exp(-2 pi i m / c)
+    for (long long c = 1; c <= N; c *= 2)
+        for (long long m = 0; m < c; ++m) {
+            double ang = -2.0 * kPi * (double)m / (double)c;
+            out[c - 1 + m].x = (decltype(out[0].x))cos(ang);
+            out[c - 1 + m].y = (decltype(out[0].x))sin(ang);
+        }
+}
+
+// exact c_N[i] = sum_j r[j%3] W_N^{ij}: one geometric series per residue class t = j % 3,
+//   S_t = W^{it} (1 - q^{n_t}) / (1 - q),  q = W^{3i},
+// with 1 - exp(-2ia) = 2i sin(a) exp(-ia) and all angles reduced in integers.
+void checksum_exact(long long N, double* re, double* im) {
+    const double rx[3] = {1.0, -0.5, -0.5}, ry[3] = {0.0, -kSqrt3_2_literal, kSqrt3_2_literal};
+    for (long long i = 0; i < N; ++i) {
+        double sx = 0, sy = 0;
+        for (int t = 0; t < 3; ++t) {
+            long long nt = (N - t + 2) / 3;              // # of j < N with j % 3 == t
+            if (nt <= 0) continue;
+            double gx, gy;                               // sum_m q^m, m < nt
+            long long q3 = (3 * i) % N;
+            if (q3 == 0) {
+                gx = (double)nt; gy = 0;
+            } else {
+                double a = kPi * (double)q3 / (double)N;
+                long long qb = (q3 * nt) % N;
+                double b = kPi * (double)qb / (double)N;
+                double mag = sin(b) / sin(a);
+                double ph = -(b - a);
+                gx = mag * cos(ph); gy = mag * sin(ph);
+            }
+            long long it = (i * t) % N;
+            double wa = -2.0 * kPi * (double)it / (double)N;
+            double wx = cos(wa), wy = sin(wa);
+            double tx = gx * wx - gy * wy, ty = gx * wy + gy * wx;
+            sx += tx * rx[t] - ty * ry[t];
+            sy += tx * ry[t] + ty * rx[t];
+        }
+        re[i] = sx; im[i] = sy;
+    }
+}
+
+// abft.h:21-61 verbatim arithmetic: angle 2*pi*i*j rounded to float before the
+// division by float(N); cos/sin and the accumulation in T.
+template <class C, class R>
+void checksum_reference(long long N, C* dest) {
+    C r[3];
+    r[0].x = (R)1.0; r[0].y = (R)0.0;
+    r[1].x = (R)-0.5; r[1].y = (R)-kSqrt3_2_literal;
+    r[2].x = (R)-0.5; r[2].y = (R)kSqrt3_2_literal;
+    for (long long i = 0; i < N; ++i) {
+        dest[i].x = 0; dest[i].y = 0;
+        for (long long j = 0; j < N; ++j) {
+            float ang = -(float)(2 * kPi * (double)i * (double)j) / (float)N;
+            R x, y;
+            if (sizeof(R) == 4) { x = (R)cosf(ang); y = (R)sinf(ang); }
+            else { x = (R)cos((double)ang); y = (R)sin((double)ang); }
+            dest[i].x += x * r[j % 3].x - y * r[j % 3].y;
+            dest[i].y += x * r[j % 3].y + y * r[j % 3].x;
+        }
+    }
+}
+
+struct c32 { float x, y; };
+struct c64 { double x, y; };
+
+}  // namespace
+
+struct turbofft_plan {
+    int logN = 0, datatype = 0, if_ft = 0, if_err = 0, thread_bs = 1;
+    Row row{};
+    int launches = 0;
+    const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
+    int tb_gap[3] = {1, 1, 1};
+    size_t esize = 8;
+    // device tables
+    void* tw = nullptr;          // concatenated twiddle table, 2*tw_N - 1 entries
+    long long tw_N = 0;
+    void* tw_lo[3] = {nullptr, nullptr, nullptr};
+    int lo_bits[3] = {0, 0, 0};
+    void* cksum[3] = {nullptr, nullptr, nullptr};
+    unsigned long long* counters = nullptr;   // 8 x u64
+    long long* flagged = nullptr;
+    int flagged_cap = 4096;
+    // FT run-time parameters
+    double err_smoothing = 1000.0, err_threshold = 1e-3;
+    int correct = 0;
+    int inj_mode = 0, inj_launch = -1, inj_every = 1, inj_s = 0, inj_m = 0;
+    long long inj_tile = 0;
+    double inj_mag = 100.0;
+    int cksum_mode = 0;
+};
+
+extern "C" {
+
+const char* turbofft_last_error(void) { return g_err.c_str(); }
+
+int turbofft_build_twiddle_table(int datatype, long long N, void* out) {
+    if (!out || N < 1 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "twiddle table: N must be a power of two");
+    if (datatype == TURBOFFT_FP32) fill_twiddle((c32*)out, N);
+    else if (datatype == TURBOFFT_FP64) fill_twiddle((c64*)out, N);
+    else return fail(TURBOFFT_EINVAL, "bad datatype %d", datatype);
+    return TURBOFFT_OK;
+}
+
+int turbofft_build_checksum_vector(int datatype, long long N, int mode, void* out) {
+    if (!out || N < 2 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "checksum vector: N must be a power of two >= 2");
+    if (datatype != TURBOFFT_FP32 && datatype != TURBOFFT_FP64) return fail(TURBOFFT_EINVAL, "bad datatype %d", datatype);
+    if (mode == 1) {
+        if (datatype == TURBOFFT_FP32) checksum_reference<c32, float>(N, (c32*)out);
+        else checksum_reference<c64, double>(N, (c64*)out);
+        return TURBOFFT_OK;
+    }
+    if (mode != 0) return fail(TURBOFFT_EINVAL, "checksum mode must be 0 (exact) or 1 (reference)");
+    std::vector<double> re(N), im(N);
+    checksum_exact(N, re.data(), im.data());
+    for (long long i = 0; i < N; ++i) {
+        if (datatype == TURBOFFT_FP32) { ((c32*)out)[i].x = (float)re[i]; ((c32*)out)[i].y = (float)im[i]; }
+        else { ((c64*)out)[i].x = re[i]; ((c64*)out)[i].y = im[i]; }
+    }
+    return TURBOFFT_OK;
+}
+
+int turbofft_builtin_plan_row(int datatype, int logN, int row[11]) {
+    if (datatype != TURBOFFT_FP32 && datatype != TURBOFFT_FP64) return fail(TURBOFFT_EINVAL, "bad datatype %d", datatype);
+    std::istringstream in(tfft_builtin_param_csv(datatype));
+    std::vector<Row> rows;
+    if (!parse_csv(in, rows)) return fail(TURBOFFT_ENOPLAN, "built-in plan table is malformed");
+    if (logN < 0 || logN >= (int)rows.size() || rows[logN].launches() == 0)
+        return fail(TURBOFFT_ENOPLAN, "no built-in plan row for logN=%d", logN);
+    memcpy(row, rows[logN].v, sizeof(int) * 11);
+    return TURBOFFT_OK;
+}
+
+int turbofft_kernel_count(void) {
+    int c = 0;
+    tfft_kernel_table(&c);
+    return c;
+}
+
+const char* turbofft_kernel_name(int i) {
+    int c = 0;
+    const tfft_kernel_entry* t = tfft_kernel_table(&c);
+    return (i >= 0 && i < c) ? t[i].name : nullptr;
+}
+
+void turbofft_plan_destroy(turbofft_plan_t* p) {
+    if (!p) return;
+    if (p->tw) (void)hipFree(p->tw);
+    for (int i = 0; i < 3; ++i) {
+        if (p->tw_lo[i]) (void)hipFree(p->tw_lo[i]);
+        if (p->cksum[i]) (void)hipFree(p->cksum[i]);
+    }
+    if (p->counters) (void)hipFree(p->counters);
+    if (p->flagged) (void)hipFree(p->flagged);
+    delete p;
+}
+
+static int plan_build(turbofft_plan* p, const char* param_csv) {
+    std::vector<Row> rows;
+    if (param_csv) {
+        std::ifstream f(param_csv);
+        if (!f.is_open()) return fail(TURBOFFT_ENOPLAN, "Failed to open file. (%s)", param_csv);   // readCSV.h:29-31
+        if (!parse_csv(f, rows)) return fail(TURBOFFT_ENOPLAN, "malformed plan CSV %s", param_csv);
+    } else {
+        std::istringstream in(tfft_builtin_param_csv(p->datatype));
+        if (!parse_csv(in, rows)) return fail(TURBOFFT_ENOPLAN, "built-in plan table is malformed");
+    }
+    if (p->logN < 1 || p->logN >= (int)rows.size() || rows[p->logN].launches() < 1 || rows[p->logN].launches() > 3)
+        return fail(TURBOFFT_ENOPLAN, "no plan row for logN=%d", p->logN);
+    p->row = rows[p->logN];
+    const Row& r = p->row;
+    if (r.logN() != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row %d describes logN=%d", p->logN, r.logN());
+    p->launches = r.launches();
+    int sum = 0;
+    for (int i = 0; i < p->launches; ++i) sum += r.logNi(i);
+    if (sum != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row for logN=%d: digit sizes sum to %d", p->logN, sum);
+    p->esize = p->datatype == TURBOFFT_FP32 ? 8 : 16;
+
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+
+    long long twN = 1;
+    for (int i = 0; i < p->launches; ++i) {
+        int kind = kind_of_launch(p->launches, i);
+        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft);
+        if (!k)
+            return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d)",
+                        i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft);
+        p->k[i] = k;
+        if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
+            HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
+        int nb = 0;
+        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k->func, k->threads, k->lds_bytes));
+        if (nb < 1) return fail(TURBOFFT_ENOPLAN, "kernel %s does not fit on a CU (LDS %d B)", k->name, k->lds_bytes);
+        p->tb_gap[i] = nb * prop.multiProcessorCount;      // fft_codegen.py:216-218 with measured residency
+        if ((1ll << r.logNi(i)) > twN) twN = 1ll << r.logNi(i);
+        if (kind == 1) {
+            // inter-launch twiddle W_(2^L)^e, L = log2(Ni * ncols): e = hi << lo_bits | lo
+            int L = 0;
+            for (int j = i; j < p->launches; ++j) L += r.logNi(j);
+            p->lo_bits[i] = (L + 1) / 2;
+            long long hiN = 1ll << (L - p->lo_bits[i]);
+            if (hiN > twN) twN = hiN;
+            if ((1 << r.logNi(i)) * (long long)r.BS(i) < 1) return fail(TURBOFFT_EINVAL, "bad tile");
+        }
+    }
+    // tile shape constraints
+    for (int i = 0; i < p->launches; ++i) {
+        int kind = kind_of_launch(p->launches, i);
+        if (kind == 1) {
+            int log_ncols = 0;
+            for (int j = i + 1; j < p->launches; ++j) log_ncols += r.logNi(j);
+            if (r.BS(i) > (1 << log_ncols)) return fail(TURBOFFT_ENOPLAN, "launch %d: BS %d exceeds %d columns", i, r.BS(i), 1 << log_ncols);
+        } else if (kind == 2) {
+            if (r.BS(i) > (1 << r.logNi(0))) return fail(TURBOFFT_ENOPLAN, "launch %d: BS %d exceeds the %d rows of the outer digit", i, r.BS(i), 1 << r.logNi(0));
+        }
+    }
+    p->tw_N = twN;
+    {
+        std::vector<char> host((size_t)(2 * twN) * p->esize);
+        turbofft_build_twiddle_table(p->datatype, twN, host.data());
+        HIP_TRY(hipMalloc(&p->tw, host.size()));
+        HIP_TRY(hipMemcpy(p->tw, host.data(), (size_t)(2 * twN - 1) * p->esize, hipMemcpyHostToDevice));
+    }
+    for (int i = 0; i < p->launches; ++i) {
+        if (kind_of_launch(p->launches, i) == 1) {
+            int L = 0;
+            for (int j = i; j < p->launches; ++j) L += r.logNi(j);
+            long long cnt = 1ll << p->lo_bits[i];
+            std::vector<char> host((size_t)cnt * p->esize);
+            for (long long l = 0; l < cnt; ++l) {
+                double ang = -2.0 * kPi * (double)l / (double)(1ll << L);
+                if (p->datatype == TURBOFFT_FP32) { ((c32*)host.data())[l].x = (float)cos(ang); ((c32*)host.data())[l].y = (float)sin(ang); }
+                else { ((c64*)host.data())[l].x = cos(ang); ((c64*)host.data())[l].y = sin(ang); }
+            }
+            HIP_TRY(hipMalloc(&p->tw_lo[i], host.size()));
+            HIP_TRY(hipMemcpy(p->tw_lo[i], host.data(), host.size(), hipMemcpyHostToDevice));
+        }
+        if (p->if_ft) {
+            long long Ni = 1ll << r.logNi(i);
+            std::vector<char> host((size_t)Ni * p->esize);
+            int rc = turbofft_build_checksum_vector(p->datatype, Ni, p->cksum_mode, host.data());
+            if (rc) return rc;
+            HIP_TRY(hipMalloc(&p->cksum[i], host.size()));
+            HIP_TRY(hipMemcpy(p->cksum[i], host.data(), host.size(), hipMemcpyHostToDevice));
+        }
+    }
+    if (p->if_ft) {
+        HIP_TRY(hipMalloc((void**)&p->counters, 8 * sizeof(unsigned long long)));
+        HIP_TRY(hipMemset(p->counters, 0, 8 * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void**)&p->flagged, sizeof(long long) * 2 * p->flagged_cap));
+        HIP_TRY(hipMemset(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap));
+    }
+    return TURBOFFT_OK;
+}
+
+turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_err, int thread_bs,
+                                      const char* param_csv) {
+    g_err.clear();
+    if (datatype != TURBOFFT_FP32 && datatype != TURBOFFT_FP64) { fail(TURBOFFT_EINVAL, "bad datatype %d", datatype); return nullptr; }
+    if (thread_bs < 1) { fail(TURBOFFT_EINVAL, "thread_bs must be >= 1"); return nullptr; }
+    turbofft_plan* p = new turbofft_plan();
+    p->logN = logN;
+    p->datatype = datatype;
+    p->if_err = if_err ? 1 : 0;
+    p->if_ft = (if_ft || if_err) ? 1 : 0;            // CommandLineParser.h:66-68
+    p->thread_bs = thread_bs;
+    if (p->if_err) { p->inj_mode = 1; p->correct = 1; }   // the if_err=1 kernels inject and correct
+    const char* env = getenv("TURBOFFT_CHECKSUM_MODE");
+    if (env && atoi(env) == 1) p->cksum_mode = 1;
+    if (plan_build(p, param_csv) != TURBOFFT_OK) {
+        std::string keep = g_err;
+        turbofft_plan_destroy(p);
+        g_err = keep;
+        return nullptr;
+    }
+    return p;
+}
+
+int turbofft_plan_info(const turbofft_plan_t* p, int* launches, int logNi[3], int BSi[3], int ni[3],
+                       size_t lds_bytes[3], int threads[3]) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (launches) *launches = p->launches;
+    for (int i = 0; i < 3; ++i) {
+        bool on = i < p->launches;
+        if (logNi) logNi[i] = on ? p->row.logNi(i) : 0;
+        if (BSi) BSi[i] = on ? p->row.BS(i) : 0;
+        if (ni) ni[i] = on ? p->row.n(i) : 0;
+        if (lds_bytes) lds_bytes[i] = on ? (size_t)p->k[i]->lds_bytes : 0;
+        if (threads) threads[i] = on ? p->k[i]->threads : 0;
+    }
+    return TURBOFFT_OK;
+}
+
+static long long launch_tiles(const turbofft_plan* p, int i, long long bs) {
+    long long tile = (1ll << p->row.logNi(i)) * p->row.BS(i);
+    long long pts = (1ll << p->logN) * bs;
+    if (p->launches == 1) return (bs + p->row.BS(0) - 1) / p->row.BS(0);
+    return pts / tile;
+}
+
+long long turbofft_plan_grid(const turbofft_plan_t* p, int launch, long long bs) {
+    if (!p || launch < 0 || launch >= p->launches || bs < 0) return fail(TURBOFFT_EINVAL, "bad argument");
+    long long nt = launch_tiles(p, launch, bs);
+    return (nt + p->thread_bs - 1) / p->thread_bs;
+}
+
+int turbofft_plan_tb_gap(const turbofft_plan_t* p, int launch) {
+    if (!p || launch < 0 || launch >= p->launches) return fail(TURBOFFT_EINVAL, "bad argument");
+    return p->tb_gap[launch];
+}
+
+int turbofft_plan_set_tb_gap(turbofft_plan_t* p, int launch, int tb_gap) {
+    if (!p || launch < 0 || launch >= p->launches || tb_gap < 1) return fail(TURBOFFT_EINVAL, "bad argument");
+    p->tb_gap[launch] = tb_gap;
+    return TURBOFFT_OK;
+}
+
+int turbofft_set_ft_params(turbofft_plan_t* p, double err_smoothing, double err_threshold, int correct) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
+    p->err_smoothing = err_smoothing;
+    p->err_threshold = err_threshold;
+    p->correct = correct ? 1 : 0;
+    return TURBOFFT_OK;
+}
+
+int turbofft_set_injection(turbofft_plan_t* p, int mode, int launch, int every, long long tile_phase, int s,
+                           int m, double mag) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
+    if (mode < 0 || mode > 2 || every < 1) return fail(TURBOFFT_EINVAL, "bad injection mode/every");
+    int li = launch < 0 ? p->launches - 1 : launch;
+    if (li >= p->launches) return fail(TURBOFFT_EINVAL, "bad injection launch");
+    if (s < 0 || s >= p->row.BS(li) || m < 0 || m >= (1 << p->row.logNi(li)))
+        return fail(TURBOFFT_EINVAL, "injection element (s=%d, m=%d) outside the tile", s, m);
+    if (mode == 2 && (tile_phase < 0 || tile_phase >= every)) return fail(TURBOFFT_EINVAL, "tile_phase must be in [0, every)");
+    p->inj_mode = mode; p->inj_launch = launch; p->inj_every = every; p->inj_tile = tile_phase;
+    p->inj_s = s; p->inj_m = m; p->inj_mag = mag;
+    return TURBOFFT_OK;
+}
+
+int turbofft_reset_ft_counters(turbofft_plan_t* p) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (!p->if_ft) return TURBOFFT_OK;
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemset(p->counters, 0, 8 * sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap));
+    return TURBOFFT_OK;
+}
+
+int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, unsigned long long* detected,
+                             unsigned long long* corrected, unsigned long long* uncorrectable,
+                             long long* flagged, int cap, int* nflagged) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    unsigned long long c[8] = {0};
+    if (p->if_ft) {
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipMemcpy(c, p->counters, sizeof c, hipMemcpyDeviceToHost));
+    }
+    if (checked) *checked = c[0];
+    if (detected) *detected = c[1];
+    if (corrected) *corrected = c[2];
+    if (uncorrectable) *uncorrectable = c[3];
+    int n = (int)(c[4] < (unsigned long long)p->flagged_cap ? c[4] : (unsigned long long)p->flagged_cap);
+    if (n > cap) n = cap < 0 ? 0 : cap;
+    if (nflagged) *nflagged = n;
+    if (flagged && n > 0) HIP_TRY(hipMemcpy(flagged, p->flagged, sizeof(long long) * 2 * n, hipMemcpyDeviceToHost));
+    return TURBOFFT_OK;
+}
+
+int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
+    if (bs == 0) return TURBOFFT_OK;
+    if (!in_d || !out_d) return fail(TURBOFFT_EINVAL, "null buffer");
+    const long long N = 1ll << p->logN;
+    if (N * bs > (1ll << 40)) return fail(TURBOFFT_EINVAL, "problem too large");
+    const Row& r = p->row;
+    char* out = (char*)out_d;
+    char* work = out + (size_t)N * bs * p->esize;
+    // ping-pong so that the last launch writes out[0 .. N*bs)
+    const void* src[3];
+    void* dst[3];
+    if (p->launches == 1) { src[0] = in_d; dst[0] = out; }
+    else if (p->launches == 2) { src[0] = in_d; dst[0] = work; src[1] = work; dst[1] = out; }
+    else { src[0] = in_d; dst[0] = out; src[1] = out; dst[1] = work; src[2] = work; dst[2] = out; }
+    for (int i = 0; i < p->launches; ++i) {
+        const tfft_kernel_entry* k = p->k[i];
+        tfft_kargs a;
+        memset(&a, 0, sizeof a);
+        a.ntiles = launch_tiles(p, i, bs);
+        a.nrows = bs;
+        a.thread_bs = p->thread_bs;
+        a.tb_gap = p->tb_gap[i];
+        int kind = kind_of_launch(p->launches, i);
+        if (kind == 1) {
+            int log_ncols = 0;
+            for (int j = i + 1; j < p->launches; ++j) log_ncols += r.logNi(j);
+            a.log_ncols = log_ncols;
+            a.tw_lo_bits = p->lo_bits[i];
+            int L = r.logNi(i) + log_ncols;
+            long long hiN = 1ll << (L - p->lo_bits[i]);
+            a.tw_hi = (const char*)p->tw + (size_t)(hiN - 1) * p->esize;
+            a.tw_lo = p->tw_lo[i];
+        } else if (kind == 2) {
+            a.logN = p->logN;
+            a.logC = r.logNi(0);
+            a.logQ = p->launches == 3 ? r.logNi(1) : 0;
+        }
+        if (p->if_ft) {
+            a.ft.cksum = p->cksum[i];
+            a.ft.counters = p->counters;
+            a.ft.flagged = p->flagged;
+            a.ft.flagged_cap = p->flagged_cap;
+            a.ft.launch = i;
+            a.ft.correct = p->correct;
+            int inj_l = p->inj_launch < 0 ? p->launches - 1 : p->inj_launch;
+            a.ft.inj_mode = (inj_l == i) ? p->inj_mode : 0;
+            a.ft.inj_every = p->inj_every;
+            a.ft.inj_tile = p->inj_tile;
+            a.ft.inj_s = p->inj_s;
+            a.ft.inj_m = p->inj_m;
+            a.ft.inj_mag = p->inj_mag;
+            a.ft.err_smoothing = p->err_smoothing;
+            a.ft.err_threshold = p->err_threshold;
+        }
+        long long grid = (a.ntiles + p->thread_bs - 1) / p->thread_bs;
+        if (grid < 1) continue;
+        if (grid > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "grid of %lld blocks exceeds the launch limit", grid);
+        const void* in_arg = src[i];
+        void* out_arg = dst[i];
+        const void* tw_arg = p->tw;
+        void* args[4] = {(void*)&in_arg, (void*)&out_arg, (void*)&tw_arg, (void*)&a};
+        HIP_TRY(hipLaunchKernel(k->func, dim3((unsigned)grid), dim3((unsigned)k->threads), args, (size_t)k->lds_bytes,
+                                (hipStream_t)stream));
+    }
+    return TURBOFFT_OK;
+}
+
+int turbofft_exec_host(turbofft_plan_t* p, const void* in_h, void* out_h, long long bs) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
+    if (bs == 0) return TURBOFFT_OK;
+    if (!in_h || !out_h) return fail(TURBOFFT_EINVAL, "null buffer");
+    size_t bytes = ((size_t)1 << p->logN) * (size_t)bs * p->esize;
+    void *in_d = nullptr, *out_d = nullptr;
+    if (hipMalloc(&in_d, bytes) != hipSuccess) return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes);
+    if (hipMalloc(&out_d, bytes * (p->launches > 1 ? 2 : 1)) != hipSuccess) {
+        (void)hipFree(in_d);
+        return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes * 2);
+    }
+    int rc = TURBOFFT_OK;
+    hipError_t e = hipMemcpy(in_d, in_h, bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        rc = turbofft_exec(p, in_d, out_d, bs, nullptr);
+        if (rc == TURBOFFT_OK) e = hipDeviceSynchronize();
+        if (rc == TURBOFFT_OK && e == hipSuccess) e = hipMemcpy(out_h, out_d, bytes, hipMemcpyDeviceToHost);
+    }
+    (void)hipFree(in_d);
+    (void)hipFree(out_d);
+    if (rc != TURBOFFT_OK) return rc;
+    if (e != hipSuccess) return fail(TURBOFFT_EHIP, "HIP error: %s", hipGetErrorString(e));
+    return TURBOFFT_OK;
+}
+
+int turbofft_time(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
+                  void* stream, float* ms_per_exec) {
+    if (!p || !ms_per_exec || reps < 1 || warmup < 0) return fail(TURBOFFT_EINVAL, "bad argument");
+    hipStream_t st = (hipStream_t)stream;
+    for (int i = 0; i < warmup; ++i) {
+        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
+        if (rc) return rc;
+    }
+    hipEvent_t t0, t1;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    HIP_TRY(hipEventRecord(t0, st));
+    for (int i = 0; i < reps; ++i) {
+        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
+        if (rc) { (void)hipEventDestroy(t0); (void)hipEventDestroy(t1); return rc; }
+    }
+    HIP_TRY(hipEventRecord(t1, st));
+    HIP_TRY(hipEventSynchronize(t1));
+    float ms = 0;
+    HIP_TRY(hipEventElapsedTime(&ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    *ms_per_exec = ms / reps;
+    return TURBOFFT_OK;
+}
+
+}  // extern "C"
