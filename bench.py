@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched FFT hot path on one MI355X.
+
+Default workload: BASELINE config 2 -- forward C2C FFT, fp32 complex, N=2^13,
+batch 2^15 (logBS+logN=28, 2 GiB in, 2 GiB out), synthetic uniform[-1,1) data
+resident in HBM before the timed region.  A "step" is one transform of the
+whole batch.  Prints ONE JSON line:
+  metric/value : algorithmic HBM GB/s = 2*N*bs*sizeof(T)/t  (the reference's
+                 figure, main.cu:69), plus "gflops" = 5*N*log2N*bs/t (main.cu:68)
+  roofline     : dominant kernel against the 8 TB/s HBM peak, timed with HIP
+                 events on the launch stream over the timed region
+  cpu_baseline : scipy.fft (pocketfft) on the host cores for a bounded sample
+                 of the same workload, scaled to the same unit
+
+Other workloads for tuning: --logN/--datatype/--bs, --sweep (logN 7..24 at
+logBS+logN=28 for both types, one JSON line per case to --out).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def make_input(torch, bs, N, datatype, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    rdt = torch.float32 if datatype == 0 else torch.float64
+    x = torch.rand((bs, N, 2), generator=g, device="cuda", dtype=rdt) * 2 - 1
+    return torch.view_as_complex(x)
+
+
+def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if_err=0, thread_bs=1, param=None,
+             x=None, out=None):
+    N = 1 << logN
+    plan = turbofft_amd.TurboFFT(logN, datatype, if_ft=if_ft, if_err=if_err, thread_bs=thread_bs, param_csv=param)
+    cdt = torch.complex64 if datatype == 0 else torch.complex128
+    if x is None:
+        x = make_input(torch, bs, N, datatype)
+    if out is None:
+        out = torch.empty(plan.out_elems(bs), dtype=cdt, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(warmup):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1000.0 / steps
+    ev_ms = ev0.elapsed_time(ev1) / steps
+    res = {
+        "logN": logN, "datatype": datatype, "bs": bs, "launches": plan.launches,
+        "plan": {"logNi": plan.logNi, "BS": plan.BS, "n": plan.n, "threads": plan.threads, "lds_bytes": plan.lds_bytes},
+        "wall_ms": wall_ms, "event_ms": ev_ms,
+        "gbs": plan.gbs(bs, wall_ms), "gflops": plan.gflops(bs, wall_ms),
+        "alg_bytes": plan.algorithmic_bytes(bs),
+    }
+    if if_ft:
+        res["ft"] = {k: v for k, v in plan.ft_counters().items() if k != "flagged"}
+    plan.close()
+    return res, x, out
+
+
+def cpu_baseline(logN, datatype, target_s=10.0):
+    """Reference CPU path: pocketfft via scipy.fft on all host cores the box
+    gives one GPU (16), on a bounded sample of the workload."""
+    import numpy as np
+    import scipy.fft
+    from oracle import turbofft_oracle as O  # noqa: F401  (the oracle's FFT is numpy/pocketfft itself)
+    N = 1 << logN
+    cores = max(1, min(16, os.cpu_count() or 1))
+    cdt = np.complex64 if datatype == 0 else np.complex128
+    rng = np.random.default_rng(0)
+    nb = max(1, (1 << 22) // N)                   # 4M points per call
+    x = (rng.uniform(-1, 1, (nb, N)) + 1j * rng.uniform(-1, 1, (nb, N))).astype(cdt)
+    scipy.fft.fft(x, axis=-1, workers=cores)      # warm-up
+    t0 = time.perf_counter()
+    calls = 0
+    while True:
+        scipy.fft.fft(x, axis=-1, workers=cores)
+        calls += 1
+        el = time.perf_counter() - t0
+        if el >= target_s or calls >= 200:
+            break
+    pts = calls * nb * N
+    esize = 8 if datatype == 0 else 16
+    gbs = 2 * pts * esize / el / 1e9
+    return {"value": gbs, "unit": "GB/s", "cores": cores, "kind": "port",
+            "gflops": 5.0 * pts * logN / el / 1e9,
+            "sample": f"scipy.fft.fft (pocketfft, workers={cores}) on {calls} x ({nb} x 2^{logN}) "
+                      f"{'complex64' if datatype == 0 else 'complex128'} transforms, {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--logN", type=int, default=13)
+    ap.add_argument("--datatype", type=int, default=0)
+    ap.add_argument("--bs", type=int, default=0, help="default 2^(28-logN)")
+    ap.add_argument("--if_ft", type=int, default=0)
+    ap.add_argument("--if_err", type=int, default=0)
+    ap.add_argument("--thread_bs", type=int, default=1)
+    ap.add_argument("--param", type=str, default=None)
+    ap.add_argument("--no_cpu", action="store_true")
+    ap.add_argument("--cpu_seconds", type=float, default=10.0)
+    ap.add_argument("--sweep", action="store_true")
+    ap.add_argument("--sweep_lo", type=int, default=7)
+    ap.add_argument("--sweep_hi", type=int, default=24)
+    ap.add_argument("--out", type=str, default=None)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (batches shard trivially across "
+              "GPUs; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        return 2
+    import torch
+    import turbofft_amd
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 1
+    if a.sweep:
+        lines = []
+        for dt in (0, 1):
+            x = out = None
+            for logN in range(a.sweep_lo, a.sweep_hi + 1):
+                bs = 1 << (28 - logN)
+                if x is not None:
+                    x = x.view(-1).view(bs, 1 << logN)
+                try:
+                    r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err,
+                                         a.thread_bs, a.param, x, out)
+                except Exception as e:   # a missing kernel for one row must not stop the sweep
+                    r = {"logN": logN, "datatype": dt, "error": str(e)}
+                if "gbs" in r:
+                    r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
+                    print(f"{'fp32' if dt == 0 else 'fp64'} logN={logN:2d} L={r['launches']} "
+                          f"{r['wall_ms']:8.3f} ms {r['gflops']:9.1f} GFLOPS {r['gbs']:8.1f} GB/s  "
+                          f"{100 * r['frac_hbm']:5.1f}% of HBM peak  {r['plan']}", flush=True)
+                else:
+                    print(r, flush=True)
+                lines.append(r)
+            del x, out
+            torch.cuda.empty_cache()
+        if a.out:
+            with open(a.out, "w") as f:
+                for r in lines:
+                    f.write(json.dumps(r) + "\n")
+        return 0
+
+    logN, dt = a.logN, a.datatype
+    bs = a.bs or (1 << (28 - logN))
+    r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err, a.thread_bs, a.param)
+    del x, out
+    tname = "fp32" if dt == 0 else "fp64"
+    launches = r["launches"]
+    # dominant kernel: with one launch it is the whole step; with several, the launches are
+    # equal-traffic passes and the per-launch average is event time / launches
+    kernel_ms = r["event_ms"] / launches
+    achieved = r["alg_bytes"] / (kernel_ms * 1e-3) / 1e9
+    line = {
+        "metric": "batched C2C FFT algorithmic HBM GB/s (2*N*bs*sizeof(T)/t) at logBS+logN=28",
+        "value": r["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": r["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if dt == 0 else "f64", "data": "synthetic",
+        "gflops": r["gflops"],
+        "config": {"workload": f"forward C2C FFT {tname} N=2^{logN} batch=2^{int(math.log2(bs))} "
+                               f"({launches}-launch plan {r['plan']['logNi']}, BS {r['plan']['BS']}, n {r['plan']['n']})"
+                               + (", fault tolerant" if a.if_ft else ""),
+                   "logN": logN, "bs": bs, "if_ft": a.if_ft, "if_err": a.if_err, "thread_bs": a.thread_bs},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel_ms": kernel_ms, "alg_bytes_per_launch": r["alg_bytes"]},
+    }
+    if a.if_ft:
+        line["ft"] = r.get("ft")
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(logN, dt, a.cpu_seconds)
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

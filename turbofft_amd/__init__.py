@@ -45,6 +45,12 @@ def lib() -> C.CDLL:
         return _lib
     if not os.path.exists(LIB_PATH):
         raise TurboFFTError(f"{LIB_PATH} is missing: run `python turbofft_amd/build.py` (there is no CPU fallback)")
+    try:
+        # PyTorch ships its own HIP runtime; when both live in one process it has to
+        # be the one that is loaded first, or torch.cuda stops seeing the device.
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH)
     vp, ll, i = C.c_void_p, C.c_longlong, C.c_int
     L.turbofft_last_error.restype = C.c_char_p
