@@ -45,6 +45,9 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
         x = make_input(torch, bs, N, datatype)
     if out is None:
         out = torch.empty(plan.out_elems(bs), dtype=cdt, device="cuda")
+    if out.numel() < plan.out_elems(bs) or x.numel() < bs * N:
+        raise ValueError(f"buffers too small for logN={logN} bs={bs}: out holds {out.numel()} elements, "
+                         f"the plan needs {plan.out_elems(bs)}")
     stream = torch.cuda.current_stream().cuda_stream
     for _ in range(warmup):
         plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
@@ -92,7 +95,7 @@ def cpu_baseline(logN, datatype, target_s=10.0):
         scipy.fft.fft(x, axis=-1, workers=cores)
         calls += 1
         el = time.perf_counter() - t0
-        if el >= target_s or calls >= 200:
+        if el >= target_s or calls >= 1000000:
             break
     pts = calls * nb * N
     esize = 8 if datatype == 0 else 16
@@ -121,6 +124,9 @@ def main():
     ap.add_argument("--sweep_lo", type=int, default=7)
     ap.add_argument("--sweep_hi", type=int, default=24)
     ap.add_argument("--out", type=str, default=None)
+    ap.add_argument("--calib_copy", type=int, default=0,
+                    help="also run this many plain device copies of the input (a kernel of known traffic, "
+                         "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (batches shard trivially across "
@@ -134,7 +140,11 @@ def main():
     if a.sweep:
         lines = []
         for dt in (0, 1):
-            x = out = None
+            # one input of 2^28 points and one output of 2*2^28 (result + workspace of the
+            # multi-launch plans) serve every logN of the sweep
+            cdt = torch.complex64 if dt == 0 else torch.complex128
+            x = make_input(torch, 1 << (28 - a.sweep_lo), 1 << a.sweep_lo, dt)
+            out = torch.empty(2 << 28, dtype=cdt, device="cuda")
             for logN in range(a.sweep_lo, a.sweep_hi + 1):
                 bs = 1 << (28 - logN)
                 if x is not None:
@@ -142,7 +152,11 @@ def main():
                 try:
                     r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err,
                                          a.thread_bs, a.param, x, out)
-                except Exception as e:   # a missing kernel for one row must not stop the sweep
+                except turbofft_amd.TurboFFTError as e:
+                    # a plan row without a compiled kernel must not stop the sweep; anything
+                    # that comes from the device does
+                    if "no compiled kernel" not in str(e) and "no plan row" not in str(e):
+                        raise
                     r = {"logN": logN, "datatype": dt, "error": str(e)}
                 if "gbs" in r:
                     r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
@@ -163,6 +177,9 @@ def main():
     logN, dt = a.logN, a.datatype
     bs = a.bs or (1 << (28 - logN))
     r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err, a.thread_bs, a.param)
+    for _ in range(a.calib_copy):
+        out.view(-1)[: x.numel()].copy_(x.view(-1))          # reads and writes x.numel()*sizeof(T) bytes
+    torch.cuda.synchronize()
     del x, out
     tname = "fp32" if dt == 0 else "fp64"
     launches = r["launches"]
