@@ -1,0 +1,101 @@
+"""Fault-tolerance path of the generated kernels, run in the CPU lock-step
+flavour: detection, location, recompute-correction, injection cadence and the
+counters, against the oracle's model of the reference checksum scheme."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import turbofft_oracle as O
+from tests import simlib
+from turbofft_amd.codegen.fft_codegen import KernelSpec
+from turbofft_amd.codegen.plan import KernelKey
+
+
+def rnd(shape, seed):
+    rng = np.random.default_rng(seed)
+    return rng.uniform(-1, 1, shape) + 1j * rng.uniform(-1, 1, shape)
+
+
+def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0,
+           inj_m=0, mag=100.0, seed=0):
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 1))
+    N = 1 << logNi
+    bs = ntiles * BS
+    x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = ntiles, bs, thread_bs, tb_gap
+    counters = np.zeros(8, dtype=np.uint64)
+    flagged = np.full(2 * 64, -7, dtype=np.int64)
+    ka.ft.counters = counters.ctypes.data
+    ka.ft.flagged = flagged.ctypes.data
+    ka.ft.flagged_cap = 64
+    ka.ft.launch = 0
+    ka.ft.correct = correct
+    ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_s, ka.ft.inj_m, ka.ft.inj_mag = \
+        inj_mode, inj_every, inj_tile, inj_s, inj_m, mag
+    ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
+    grid = (ntiles + thread_bs - 1) // thread_bs
+    ck = O.dft_checksum_vector(N, dtype)
+    y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
+    nfl = int(counters[4])
+    fl = [(int(flagged[2 * i]), int(flagged[2 * i + 1])) for i in range(min(nfl, 64))]
+    return sp, x, y, counters, fl
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+def test_clean_run_detects_nothing(dtype):
+    sp, x, y, c, fl = run_ft(dtype, 8, 4, 16, 24, 4, 3, inj_mode=0, correct=1)
+    assert c[0] == 6 and c[1] == 0 and c[2] == 0 and not fl
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, 8)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("logNi,BS,n", [(8, 4, 16), (7, 8, 8), (10, 1, 8)])
+def test_reference_cadence_detect_locate_correct(dtype, logNi, BS, n):
+    ntiles, tbs, gap = 24, 4, 3
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=1, correct=1)
+    groups = O.tile_groups(ntiles, tbs, gap)
+    injs = O.reference_injections(groups, tbs, 100.0)
+    assert c[0] == len(groups)
+    assert c[1] == len(injs) == c[2] and c[3] == 0
+    # located tiles are exactly the injected ones (decision parity with the oracle model)
+    assert sorted(t for _, t in fl) == sorted(i.tile for i in injs)
+    xt = x.reshape(ntiles, BS, -1)
+    yt = O.fft_ref(xt).astype(simlib.ctype_of(dtype))
+    for inj in injs:
+        yt[inj.tile, inj.s, :] += inj.mag
+    dec = O.ft_launch_model(xt, yt, n, groups, dtype, O.dft_checksum_vector(1 << logNi, dtype))
+    assert sorted(d.tile for d in dec if d.detected) == sorted(t for _, t in fl)
+    # corrected output equals the clean transform
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+
+
+def test_detection_without_correction_leaves_the_error():
+    sp, x, y, c, fl = run_ft("double2", 8, 4, 16, 8, 2, 2, inj_mode=1, correct=0)
+    assert c[1] == 4 and c[2] == 0
+    err = np.abs(y - O.fft_ref(x)).reshape(8, 4, 256)
+    groups = O.tile_groups(8, 2, 2)
+    for inj in O.reference_injections(groups, 2, 100.0):
+        assert np.allclose(err[inj.tile, 0], 100.0, rtol=1e-9)      # every output of that sub-FFT is off by mag
+        assert err[inj.tile, 1:].max() < 1e-9
+
+
+def test_host_chosen_injection_single_tile():
+    # mode 2: one tile in the whole run, arbitrary element
+    ntiles, tbs, gap = 20, 5, 2
+    sp, x, y, c, fl = run_ft("float2", 8, 4, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000,
+                             inj_tile=13, inj_s=2, inj_m=77, mag=100.0)
+    assert c[1] == 1 and c[2] == 1 and fl == [(0, 13)]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("float2", 8)
+
+
+def test_injection_on_arbitrary_element_matches_model_delta():
+    # error on x[m] shifts y[k] by mag*W^{mk}; the model must see the same delta sign/size
+    ntiles, tbs, gap = 4, 4, 1
+    sp, x, y, c, fl = run_ft("double2", 7, 8, 8, ntiles, tbs, gap, inj_mode=2, correct=0, inj_every=1000,
+                             inj_tile=2, inj_s=5, inj_m=3, mag=50.0)
+    assert c[1] == 1 and fl == [(0, 2)]
+    k = np.arange(128)
+    err = (y - O.fft_ref(x)).reshape(4, 8, 128)[2, 5]
+    assert np.allclose(err, 50.0 * np.exp(-2j * np.pi * 3 * k / 128), atol=1e-9)

@@ -1,0 +1,230 @@
+"""GPU fault-tolerance parity: counters, located tiles and corrected output of
+the FT kernels against the oracle's model of the reference checksum scheme
+(same thresholds, same group formula, same injection cadence)."""
+import numpy as np
+import pytest
+
+import turbofft_amd
+from oracle import turbofft_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def cdtype(dt):
+    return np.complex64 if dt == "float2" else np.complex128
+
+
+def make(bs, N, dt, seed=0):
+    rng = np.random.default_rng(seed)
+    return (rng.uniform(-1, 1, (bs, N)) + 1j * rng.uniform(-1, 1, (bs, N))).astype(cdtype(dt))
+
+
+def run(plan, x):
+    torch = _torch()
+    print(f"[ft case] logN={plan.logN} dt={plan.datatype} bs={x.shape[0]} launches={plan.launches} Ni={plan.logNi} "
+          f"BS={plan.BS} n={plan.n} tbs={plan.thread_bs}", flush=True)
+    plan.reset_ft_counters()
+    y = plan.fft(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    return y.cpu().numpy(), plan.ft_counters()
+
+
+CASES = [("float2", 10, 64), ("double2", 10, 16), ("float2", 13, 32), ("double2", 15, 8), ("float2", 16, 4),
+         ("float2", 21, 1), ("double2", 20, 2)]
+
+
+@pytest.mark.parametrize("dt,logN,bs", CASES)
+@pytest.mark.parametrize("tbs", [1, 4])
+def test_clean_ft_run(dt, logN, bs, tbs):
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=tbs)
+    x = make(bs, 1 << logN, dt, logN)
+    y, c = run(plan, x)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    assert c["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
+    assert c["detected"] == 0 and c["corrected"] == 0 and c["flagged"] == []
+
+
+@pytest.mark.parametrize("dt,logN,bs", CASES)
+@pytest.mark.parametrize("tbs", [2, 8])
+def test_reference_cadence_matches_oracle_model(dt, logN, bs, tbs):
+    # if_err=1: every block of the last launch injects into element 0 of the tile
+    # cnt == block % thread_bs + 1, detects, locates and recomputes it.  The expected
+    # decisions come from the oracle's model of the reference scheme; the magnitude is
+    # 100 (the reference default) for the 1024-point plans; for the larger ones the model
+    # says the relative rule |delta|/(1000+|mag|) > 1e-3 does not fire at 100 on U[-1,1)
+    # data (see the next test), so they inject an error sized from the data's checksum magnitude.
+    plan = turbofft_amd.TurboFFT(logN, dt, if_err=1, thread_bs=tbs)
+    gaps = [7, 5, 3][:plan.launches]
+    for i, g in enumerate(gaps):
+        plan.set_tb_gap(i, g)
+    x = make(bs, 1 << logN, dt, logN + 1)
+    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row(dt, logN))
+    if logN <= 10:
+        mag = 100.0
+    else:
+        # the rule is relative to the checksum magnitude of the data, which grows with the
+        # tile and with every launch: size the error 30x above the rule's floor for this data
+        clean, _ = O.ft_plan_model(x, row, dt, tbs, gaps, None)
+        mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[-1])) / 0.366))
+    plan.set_injection(1, mag=mag)
+    y, c = run(plan, x)
+    geoms = O.launch_geometry(row, bs)
+    last = geoms[-1]
+    groups = O.tile_groups(last.ntiles, tbs, gaps[plan.launches - 1])
+    injs = O.reference_injections(groups, tbs, mag)
+    dec, _ = O.ft_plan_model(x, row, dt, tbs, gaps, injs)
+    # keep away from the decision boundary: reduction order differs between GPU and model
+    for dl in dec:
+        for d in dl:
+            ratio = abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3
+            assert ratio < 0.67 or ratio > 1.5, "test case sits on the detection threshold"
+    model = sorted((li, d.tile) for li, dl in enumerate(dec) for d in dl if d.detected)
+    assert model == sorted((plan.launches - 1, i.tile) for i in injs)      # every injection is caught
+    assert sorted(c["flagged"]) == model
+    assert c["detected"] == len(injs) == c["corrected"] and c["uncorrectable"] == 0
+    # corrected result is bit-identical to a run without injection
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    assert c0["detected"] == 0
+    assert np.array_equal(y, y0)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+
+
+def test_reference_default_magnitude_is_below_the_rule_at_8192_points():
+    # the model of the reference rule predicts NO detection for err_inj=100 on a
+    # U[-1,1) fp32 8192-point tile (|delta| = 36.6, mag ~ 1.5e5): the GPU must agree
+    plan = turbofft_amd.TurboFFT(13, "float2", if_err=1, thread_bs=2)
+    plan.set_tb_gap(0, 7)
+    x = make(32, 1 << 13, "float2", 14)
+    y, c = run(plan, x)
+    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row("float2", 13))
+    groups = O.tile_groups(32, 2, 7)
+    injs = O.reference_injections(groups, 2, 100.0)
+    dec, _ = O.ft_plan_model(x, row, "float2", 2, [7], injs)
+    assert not any(d.detected for d in dec[0])
+    assert c["detected"] == 0 and c["checked"] == len(groups)
+    err = np.abs(y - O.fft_ref(x))
+    for inj in injs:                      # the undetected error is still in the output
+        assert np.allclose(err[inj.tile], 100.0, rtol=1e-3)
+
+
+def test_detect_only_leaves_error_in_place():
+    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1, thread_bs=4)
+    plan.set_ft_params(1000.0, 1e-3, correct=False)
+    plan.set_injection(2, every=1 << 30, tile_phase=5, s=0, m=0, mag=100.0)
+    x = make(32, 1024, "double2", 3)
+    y, c = run(plan, x)
+    assert c["detected"] == 1 and c["corrected"] == 0 and c["flagged"] == [(0, 5)]
+    err = np.abs(y - O.fft_ref(x))
+    assert np.allclose(err[5], 100.0, rtol=1e-9) and np.delete(err, 5, axis=0).max() < 1e-9
+
+
+def test_threshold_rule():
+    # |delta| / (err_smoothing + |mag|) > err_threshold with delta = -mag_inj (Ni = 1 mod 3)
+    x = make(16, 1024, "double2", 4)
+    for mag, expect in ((0.5, 0), (100.0, 1)):      # data checksum magnitude ~1e4: floor ~11
+        plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1, thread_bs=1)
+        plan.set_injection(2, every=1 << 30, tile_phase=3, mag=mag)
+        _, c = run(plan, x)
+        assert c["detected"] == expect
+    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1, thread_bs=1)
+    plan.set_ft_params(0.0, 1e-6, correct=True)          # tight rule catches the small error too
+    plan.set_injection(2, every=1 << 30, tile_phase=3, mag=0.5)
+    y, c = run(plan, x)
+    assert c["detected"] == 1 and c["corrected"] == 1
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance("double2", 10)
+
+
+def test_injection_in_an_earlier_launch_is_caught_there():
+    plan = turbofft_amd.TurboFFT(15, "double2", if_ft=1, thread_bs=2)
+    plan.set_ft_params(1000.0, 1e-3, correct=True)
+    plan.set_injection(2, launch=0, every=1 << 30, tile_phase=9, s=3, m=17, mag=100.0)
+    x = make(4, 1 << 15, "double2", 5)
+    y, c = run(plan, x)
+    assert c["flagged"] == [(0, 9)] and c["corrected"] == 1
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance("double2", 15)
+
+
+def _model_groups_last_launch(xsel, row, dt, groups, tiles_per_transform, injs, tbs):
+    """Oracle decisions for selected tile groups of the last launch.  xsel maps a batch
+    index to that transform's input; only the transforms the groups touch are needed."""
+    cache = {}
+    geom1 = O.launch_geometry(row, 1)[-1]
+    xin, yout, remap = [], [], {}
+    for g in groups:
+        for t in g:
+            b, lt = divmod(t, tiles_per_transform)
+            if b not in cache:
+                _, stages = O.plan_fft(xsel[b][None, :], row, dt, return_stages=True)
+                cache[b] = (geom1.gather(stages[-1][0]), geom1.gather(stages[-1][1]))
+            remap[t] = len(xin)
+            xin.append(cache[b][0][lt])
+            yout.append(cache[b][1][lt].copy())
+    for inj in injs:
+        if inj.tile in remap:
+            k = np.arange(geom1.Ni)
+            yout[remap[inj.tile]][inj.s] += inj.mag * np.exp(-2j * np.pi * ((inj.m * k) % geom1.Ni) / geom1.Ni)
+    lg = [[remap[t] for t in g] for g in groups]
+    dec = O.ft_launch_model(np.stack(xin), np.stack(yout), geom1.n, lg, dt,
+                            O.dft_checksum_vector(geom1.Ni, dt))
+    return dec
+
+
+def test_config5_fp64_2p20_batch256():
+    # BASELINE config 5: fp64, N=2^20, batch 256, threshold 1e-3, err_smoothing 1000, one
+    # error in 1 of every 1000 tile groups of the last launch.  Run (i) with the stated
+    # magnitude 100 and (ii) with an error sized above the rule's floor for this data;
+    # the decisions of every group that holds an injected tile must equal the oracle model's.
+    torch = _torch()
+    logN, bs, tbs = 20, 256, 8
+    N = 1 << logN
+    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row("double2", logN))
+    plan = turbofft_amd.TurboFFT(logN, "double2", if_ft=1, thread_bs=tbs)
+    plan.set_ft_params(1000.0, 1e-3, correct=True)
+    last = plan.launches - 1
+    gap = 64
+    plan.set_tb_gap(last, gap)
+    tile_elems = (1 << plan.logNi[last]) * plan.BS[last]
+    ntiles = N * bs // tile_elems
+    tpt = N // tile_elems
+    every = 1000 * tbs
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.view_as_complex(torch.rand((bs, N, 2), generator=g, device="cuda", dtype=torch.float64) * 2 - 1)
+    groups_all = O.tile_groups(ntiles, tbs, gap)
+    inj_tiles = list(range(123, ntiles, every))
+    hit_groups = [gr for gr in groups_all if any(t in gr for t in inj_tiles)]
+    need = sorted({t // tpt for gr in hit_groups for t in gr})
+    xsel = {b: x[b].cpu().numpy() for b in need}
+    ref_idx = need[:3]
+    for mag in (100.0, None):
+        if mag is None:
+            clean = _model_groups_last_launch(xsel, row, "double2", hit_groups, tpt, [], tbs)
+            mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean)) / 1.0))
+        injs = [O.Injection(t, 1, 5, mag) for t in inj_tiles]
+        dec = _model_groups_last_launch(xsel, row, "double2", hit_groups, tpt, injs, tbs)
+        for d in dec:
+            ratio = abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3
+            assert ratio < 0.67 or ratio > 1.5, "test case sits on the detection threshold"
+        plan.set_injection(2, every=every, tile_phase=123, s=1, m=5, mag=mag)
+        plan.reset_ft_counters()
+        y = plan.fft(x)
+        torch.cuda.synchronize()
+        c = plan.ft_counters()
+        model = []
+        for d, gr in zip(dec, hit_groups):
+            if d.detected:
+                model.append((last, gr[d.k - 1] if 1 <= d.k <= len(gr) else -1))
+        print("config5 mag", mag, {k: v for k, v in c.items() if k != "flagged"}, "model detections", len(model), flush=True)
+        assert c["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
+        assert sorted(c["flagged"]) == sorted(model)
+        assert c["detected"] == len(model) == c["corrected"] and c["uncorrectable"] == 0
+        if len(model) == len(inj_tiles):         # everything corrected: transforms must be clean
+            for b in ref_idx:
+                assert O.rel_l2(y[b].cpu().numpy(), O.fft_ref(xsel[b])) <= O.tolerance("double2", logN)
+    assert len(model) == len(inj_tiles)          # the sized error is caught in every group
