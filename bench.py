@@ -109,8 +109,8 @@ def cpu_baseline(logN, datatype, target_s=10.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--logN", type=int, default=13)
     ap.add_argument("--datatype", type=int, default=0)
     ap.add_argument("--bs", type=int, default=0, help="default 2^(28-logN)")
