@@ -78,6 +78,13 @@ int turbofft_exec_host(turbofft_plan_t* plan, const void* in_h, void* out_h, lon
 int turbofft_time(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
                   int warmup, int reps, void* stream, float* ms_per_exec);
 
+/* Like turbofft_time, with HIP events around every launch of the plan:
+ * ms_per_launch[i] receives the mean duration of launch i (entries beyond the
+ * plan's launch count are set to 0).  No counterpart in the reference, which
+ * times whole plans only (main.cu:52-67). */
+int turbofft_time_launches(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
+                           int warmup, int reps, void* stream, float ms_per_launch[3]);
+
 /* Plan description: launches, per-launch log2 size, BS, n, dynamic LDS bytes,
  * threads per block (the CSV row, main.cu:8-9,22-27). */
 int turbofft_plan_info(const turbofft_plan_t* plan, int* launches, int logNi[3], int BSi[3],

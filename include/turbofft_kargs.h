@@ -44,7 +44,8 @@ typedef struct tfft_kargs {
     int logC;
     int logN;             /* rowT: log2 of the whole transform                             */
     int tw_lo_bits;       /* col : W^e = tw_hi[e >> lo_bits] * tw_lo[e & mask]             */
-    int pad0;
+    int xcd_chunk;        /* >0: blocks are renumbered so that each of the 8 XCDs (block % 8)
+                             works on chunks of this many consecutive tiles; 0: identity      */
     const void* tw_hi;
     const void* tw_lo;
     tfft_ft_args ft;

@@ -31,7 +31,7 @@ class FtArgs(C.Structure):
 class KArgs(C.Structure):
     _fields_ = [("ntiles", C.c_longlong), ("nrows", C.c_longlong), ("thread_bs", C.c_int),
                 ("tb_gap", C.c_int), ("log_ncols", C.c_int), ("logQ", C.c_int), ("logC", C.c_int),
-                ("logN", C.c_int), ("tw_lo_bits", C.c_int), ("pad0", C.c_int),
+                ("logN", C.c_int), ("tw_lo_bits", C.c_int), ("xcd_chunk", C.c_int),
                 ("tw_hi", C.c_void_p), ("tw_lo", C.c_void_p), ("ft", FtArgs)]
 
 

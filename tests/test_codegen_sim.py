@@ -87,3 +87,16 @@ def test_rowT(dtype, logA, BS, n, logQ, logC):
     xc = x.astype(simlib.ctype_of(dtype)).astype(np.complex128)
     ref = np.transpose(np.fft.fft(xc, axis=3), (0, 3, 2, 1))          # [b, ka, kb, kc]
     assert O.rel_l2(y, ref) < O.tolerance(dtype, logA)
+
+
+@pytest.mark.parametrize("chunk,bs", [(1, 37), (2, 40), (3, 100), (64, 20)])
+def test_xcd_renumbering_is_a_bijection(chunk, bs):
+    # the XCD-aware block renumbering must still visit every tile exactly once
+    sp = KernelSpec(KernelKey("float2", "row1", 9, 1, 8, 0))
+    N = 512
+    x = rnd((bs, N), 11)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap, ka.xcd_chunk = bs, bs, 1, 4, chunk
+    y = simlib.run_sim(sp, x, bs * N, ka, bs, simlib.twiddle_table(N, "float2")).reshape(bs, N)
+    assert not np.isnan(y).any()
+    assert O.rel_l2(y, O.fft_ref(x.astype(np.complex64))) < O.tolerance("float2", 9)

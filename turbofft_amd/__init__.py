@@ -61,6 +61,7 @@ def lib() -> C.CDLL:
     L.turbofft_exec.argtypes = [vp, vp, vp, ll, vp]
     L.turbofft_exec_host.argtypes = [vp, vp, vp, ll]
     L.turbofft_time.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_time_launches.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_plan_info.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i), C.POINTER(i),
                                      C.POINTER(C.c_size_t), C.POINTER(i)]
     L.turbofft_plan_grid.argtypes = [vp, i, ll]
@@ -198,6 +199,12 @@ class TurboFFT:
         ms = C.c_float()
         _check(lib().turbofft_time(self._h, in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
         return ms.value
+
+    def time_launches(self, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0):
+        """Mean duration of every launch of the plan (HIP events around each launch)."""
+        ms = (C.c_float * 3)()
+        _check(lib().turbofft_time_launches(self._h, in_ptr, out_ptr, bs, warmup, reps, stream, ms))
+        return list(ms)[: self.launches]
 
     # ---- fault tolerance ----
     def set_ft_params(self, err_smoothing: float = 1000.0, err_threshold: float = 1e-3, correct: bool = True):

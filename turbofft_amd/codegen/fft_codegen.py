@@ -328,38 +328,55 @@ class KernelEmitter:
 
     # ---------- global addressing ----------
     def emit_tile_decode(self, c: Code):
+        """Wave-uniform part of the tile's addresses (64-bit, lives in SGPRs)."""
         sp = self.s
         lBS = ilog2(sp.BS)
+        lNi = ilog2(sp.Ni)
         if sp.kind == "row1":
             c(f"const long long row0 = tile << {lBS};")
+            c(f"const long long ubase = row0 << {lNi};")
         elif sp.kind == "col":
             c(f"const unsigned tpl = (unsigned)a.log_ncols - {lBS}u;")
             c("const unsigned ct = (unsigned)(tile & ((1ll << tpl) - 1));")
             c("const long long outer = tile >> tpl;")
-            c(f"const long long tbase = (outer << ({ilog2(sp.Ni)} + a.log_ncols)) + ((long long)ct << {lBS});")
+            c(f"const long long ubase = (outer << ({lNi} + a.log_ncols)) + ((long long)ct << {lBS});")
+            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
         else:
             c(f"const unsigned ctl = (unsigned)a.logC - {lBS}u;")
             c("const unsigned ct = (unsigned)(tile & ((1ll << ctl) - 1));")
             c("const unsigned qd = (unsigned)((tile >> ctl) & ((1ll << a.logQ) - 1));")
             c("const long long tb = (tile >> (ctl + a.logQ)) << a.logN;")
+            c(f"const long long ubase_in = tb + ((long long)(qd + ((ct << {lBS}) << a.logQ)) << {lNi});")
+            c(f"const unsigned ls = (unsigned)a.logN - {lNi}u;")
+            c(f"const long long ubase_out = tb + (ct << {lBS}) + ((long long)qd << a.logC);")
+            c(f"const long long gstep = {sp.Tr}ll << ls;")
 
     def emit_load(self, c: Code):
         sp = self.s
         lNi = ilog2(sp.Ni)
         if sp.kind == "row1":
-            c(f"const long long gi = ((row0 + s) << {lNi}) + x;")
-            c("const bool ok = (row0 + s) < a.nrows;")
+            c(f"const unsigned gi = (s << {lNi}) + x;")
+            if sp.BS > 1:
+                c("if ((row0 + s) < a.nrows) {")
+                c.ind += 1
             for e in range(sp.n):
-                c(f"r[{e}] = ok ? GLD(in, gi + {sp.Tr * e}) : czero(r[0]);")
+                c(f"r[{e}] = GLDU(in, ubase + {sp.Tr * e}, gi);")
+            if sp.BS > 1:
+                c.ind -= 1
+                c("} else {")
+                c.ind += 1
+                for e in range(sp.n):
+                    c(f"r[{e}] = czero(r[0]);")
+                c.ind -= 1
+                c("}")
         elif sp.kind == "col":
-            c(f"const long long gi = tbase + s + ((long long)x << a.log_ncols);")
-            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
+            c("const unsigned gi = s + (x << a.log_ncols);")
             for e in range(sp.n):
-                c(f"r[{e}] = GLD(in, gi + {e} * gstep);")
+                c(f"r[{e}] = GLDU(in, ubase + {e} * gstep, gi);")
         else:
-            c(f"const long long gi = tb + ((long long)(qd + (((ct << {ilog2(sp.BS)}) + s) << a.logQ)) << {lNi}) + x;")
+            c(f"const unsigned gi = ((s << a.logQ) << {lNi}) + x;")
             for e in range(sp.n):
-                c(f"r[{e}] = GLD(in, gi + {sp.Tr * e});")
+                c(f"r[{e}] = GLDU(in, ubase_in + {sp.Tr * e}, gi);")
 
     def out_reg(self, e: int) -> int:
         """Register that holds output k = x + Tr*e after the last pass."""
@@ -373,26 +390,25 @@ class KernelEmitter:
         sp = self.s
         lNi = ilog2(sp.Ni)
         if sp.kind == "row1":
-            c(f"const long long go = ((row0 + s) << {lNi}) + x;")
-            c("if ((row0 + s) < a.nrows) {")
-            c.ind += 1
+            c(f"const unsigned go = (s << {lNi}) + x;")
+            if sp.BS > 1:
+                c("if ((row0 + s) < a.nrows) {")
+                c.ind += 1
             for e in range(sp.n):
-                c(f"GST(out, go + {sp.Tr * e}, r[{self.out_reg(e)}]);")
-            c.ind -= 1
-            c("}")
+                c(f"GSTU(out, ubase + {sp.Tr * e}, go, r[{self.out_reg(e)}]);")
+            if sp.BS > 1:
+                c.ind -= 1
+                c("}")
         elif sp.kind == "col":
             c("const unsigned col = (ct << %d) + s;" % ilog2(sp.BS))
             self.emit_interlaunch_twiddle(c)
-            c(f"const long long go = tbase + s + ((long long)x << a.log_ncols);")
-            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
+            c("const unsigned go = s + (x << a.log_ncols);")
             for e in range(sp.n):
-                c(f"GST(out, go + {e} * gstep, r[{self.out_reg(e)}]);")
+                c(f"GSTU(out, ubase + {e} * gstep, go, r[{self.out_reg(e)}]);")
         else:
-            c(f"const unsigned ls = (unsigned)a.logN - {lNi}u;")
-            c(f"const long long go = tb + ((ct << {ilog2(sp.BS)}) + s) + ((long long)qd << a.logC) + ((long long)x << ls);")
-            c(f"const long long gstep = {sp.Tr}ll << ls;")
+            c("const unsigned go = s + (x << ls);")
             for e in range(sp.n):
-                c(f"GST(out, go + {e} * gstep, r[{self.out_reg(e)}]);")
+                c(f"GSTU(out, ubase_out + {e} * gstep, go, r[{self.out_reg(e)}]);")
 
     def emit_interlaunch_twiddle(self, c: Code):
         """r[k] *= W_(Ni*ncols)^(col*k), k = x + Tr*e: base and step come from the
@@ -510,8 +526,9 @@ class KernelEmitter:
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
             c(f"struct TS {{ {T2} r[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
-            c("for (long long bx = 0; bx < grid; ++bx) {")
+            c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
+            c("long long bx = pbx;")
             c(f"std::vector<{T2}> ldsv({sp.lds_elems}); {T2}* lds = ldsv.data();")
             c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
         else:
@@ -522,10 +539,18 @@ class KernelEmitter:
             c("extern __shared__ __align__(16) unsigned char lds_raw[];")
             c(f"{T2}* lds = ({T2}*)lds_raw;")
             c("const unsigned tx = threadIdx.x;")
-            c("const long long bx = blockIdx.x, grid = gridDim.x;")
+            c("const long long grid = gridDim.x;")
+            c("long long bx = blockIdx.x;")
             c(f"{T2} r[{sp.n}];")
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
+        # XCD-aware renumbering: hardware deals blocks round-robin to the 8 XCDs, so block
+        # b runs on XCD b % 8.  Give every XCD chunks of `xcd_chunk` consecutive tiles (its
+        # L2 then streams contiguous memory) while the 8 XCDs stay in one neighbourhood.
+        c("if (a.xcd_chunk > 0) {")
+        c("    const long long span = 8ll * a.xcd_chunk, full = (grid / span) * span;")
+        c("    if (bx < full) { const long long q = bx >> 3, xcd = bx & 7; bx = (q / a.xcd_chunk) * span + xcd * a.xcd_chunk + q % a.xcd_chunk; }")
+        c("}")
         c(f"const {T2}* twhi = (const {T2}*)a.tw_hi; const {T2}* twlo = (const {T2}*)a.tw_lo; const {T2}* ck = (const {T2}*)a.ft.cksum;")
         c("(void)twhi; (void)twlo; (void)ck;")
         # tile group of this block (fft_codegen.py:218,260-261 with a rounded-up grid)

@@ -15,6 +15,10 @@
 #define TFFT_DEV __device__ __forceinline__
 #define GLD(p, i) ((p)[(i)])
 #define GST(p, i, v) ((p)[(i)] = (v))
+// wave-uniform 64-bit base + 32-bit per-lane offset: lets the compiler keep the base in
+// SGPRs (saddr addressing) so an access costs no vector address arithmetic
+#define GLDU(p, ub, off) (((p) + (ub))[(off)])
+#define GSTU(p, ub, off, v) (((p) + (ub))[(off)] = (v))
 #define TWLD(p, i) ((p)[(i)])
 #define LLD(i) (lds[(i)])
 #define LST(i, v) (lds[(i)] = (v))
@@ -36,6 +40,8 @@ extern long long tfft_sim_errors;
          : (long long)(i))
 #define GLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
 #define GST(p, i, v) ((p)[TFFT_CHK((i), p##_limit, #p)] = (v))
+#define GLDU(p, ub, off) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)])
+#define GSTU(p, ub, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)] = (v))
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))

@@ -181,6 +181,7 @@ struct turbofft_plan {
     long long inj_tile = 0;
     double inj_mag = 100.0;
     int cksum_mode = 0;
+    int xcd_chunk = 64;          // tiles per XCD chunk (0 = plain block order)
 };
 
 extern "C" {
@@ -363,6 +364,8 @@ turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_
     if (p->if_err) { p->inj_mode = 1; p->correct = 1; }   // the if_err=1 kernels inject and correct
     const char* env = getenv("TURBOFFT_CHECKSUM_MODE");
     if (env && atoi(env) == 1) p->cksum_mode = 1;
+    env = getenv("TURBOFFT_XCD_CHUNK");
+    if (env) p->xcd_chunk = atoi(env) > 0 ? atoi(env) : 0;
     if (plan_build(p, param_csv) != TURBOFFT_OK) {
         std::string keep = g_err;
         turbofft_plan_destroy(p);
@@ -464,7 +467,14 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
     return TURBOFFT_OK;
 }
 
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev);
+
 int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
+    return exec_impl(p, in_d, out_d, bs, stream, nullptr);
+}
+
+// ev (optional): launches+1 events; ev[i] is recorded before launch i, ev[launches] after the last
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
     if (bs == 0) return TURBOFFT_OK;
@@ -488,6 +498,7 @@ int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long b
         a.nrows = bs;
         a.thread_bs = p->thread_bs;
         a.tb_gap = p->tb_gap[i];
+        a.xcd_chunk = p->xcd_chunk;
         int kind = kind_of_launch(p->launches, i);
         if (kind == 1) {
             int log_ncols = 0;
@@ -527,10 +538,37 @@ int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long b
         void* out_arg = dst[i];
         const void* tw_arg = p->tw;
         void* args[4] = {(void*)&in_arg, (void*)&out_arg, (void*)&tw_arg, (void*)&a};
+        if (ev) HIP_TRY(hipEventRecord(ev[i], (hipStream_t)stream));
         HIP_TRY(hipLaunchKernel(k->func, dim3((unsigned)grid), dim3((unsigned)k->threads), args, (size_t)k->lds_bytes,
                                 (hipStream_t)stream));
     }
+    if (ev) HIP_TRY(hipEventRecord(ev[p->launches], (hipStream_t)stream));
     return TURBOFFT_OK;
+}
+
+int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
+                           void* stream, float ms_per_launch[3]) {
+    if (!p || !ms_per_launch || reps < 1 || warmup < 0 || bs < 1) return fail(TURBOFFT_EINVAL, "bad argument");
+    for (int i = 0; i < 3; ++i) ms_per_launch[i] = 0.f;
+    for (int i = 0; i < warmup; ++i) {
+        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
+        if (rc) return rc;
+    }
+    hipEvent_t ev[4];
+    for (int i = 0; i < 4; ++i) HIP_TRY(hipEventCreate(&ev[i]));
+    int rc = TURBOFFT_OK;
+    for (int r = 0; r < reps && rc == TURBOFFT_OK; ++r) {
+        rc = exec_impl(p, in_d, out_d, bs, stream, ev);
+        if (rc) break;
+        if (hipEventSynchronize(ev[p->launches]) != hipSuccess) { rc = fail(TURBOFFT_EHIP, "hipEventSynchronize failed"); break; }
+        for (int i = 0; i < p->launches; ++i) {
+            float ms = 0;
+            if (hipEventElapsedTime(&ms, ev[i], ev[i + 1]) != hipSuccess) { rc = fail(TURBOFFT_EHIP, "hipEventElapsedTime failed"); break; }
+            ms_per_launch[i] += ms / reps;
+        }
+    }
+    for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
+    return rc;
 }
 
 int turbofft_exec_host(turbofft_plan_t* p, const void* in_h, void* out_h, long long bs) {
