@@ -100,3 +100,86 @@ def test_xcd_renumbering_is_a_bijection(chunk, bs):
     y = simlib.run_sim(sp, x, bs * N, ka, bs, simlib.twiddle_table(N, "float2")).reshape(bs, N)
     assert not np.isnan(y).any()
     assert O.rel_l2(y, O.fft_ref(x.astype(np.complex64))) < O.tolerance("float2", 9)
+
+
+SPLIT = [("row1", "float2", 10, 1, 16), ("row1", "double2", 9, 2, 8), ("row1", "float2", 13, 1, 32), ("row1", "float2", 7, 8, 8)]
+
+
+@pytest.mark.parametrize("kind,dtype,logNi,BS,n", SPLIT)
+def test_split_exchange_row1(kind, dtype, logNi, BS, n):
+    # re and im go through a half-size LDS buffer in two rounds
+    sp = KernelSpec(KernelKey(dtype, kind, logNi, BS, n, 0, 1))
+    full = KernelSpec(KernelKey(dtype, kind, logNi, BS, n, 0, 0))
+    assert sp.lds_bytes <= full.lds_bytes // 2 + 4096
+    N = 1 << logNi
+    bs = BS * 3
+    x = rnd((bs, N), logNi + 50)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = bs // BS, bs, 2, 2
+    y = simlib.run_sim(sp, x, bs * N, ka, (ka.ntiles + 1) // 2, simlib.twiddle_table(N, dtype)).reshape(bs, N)
+    assert O.rel_l2(y, O.fft_ref(x.astype(simlib.ctype_of(dtype)))) < O.tolerance(dtype, logNi)
+
+
+def test_split_exchange_col_and_rowT():
+    dtype = "float2"
+    sp = KernelSpec(KernelKey(dtype, "col", 8, 16, 16, 0, 1))
+    Ni, ncols, outer, log_ncols = 256, 64, 2, 6
+    x = rnd((outer, Ni, ncols), 5)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.thread_bs, ka.tb_gap, ka.log_ncols = outer * ncols // 16, 1, 3, log_ncols
+    lo_bits, hi, lo = simlib.split_tables(8 + log_ncols, dtype)
+    ka.tw_lo_bits = lo_bits
+    y = simlib.run_sim(sp, x, x.size, ka, ka.ntiles, simlib.twiddle_table(Ni, dtype), hi, lo).reshape(outer, Ni, ncols)
+    ref = np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=1)
+    ref = ref * np.exp(-2j * np.pi * ((np.arange(Ni)[:, None] * np.arange(ncols)[None, :]) % (Ni * ncols)) / (Ni * ncols))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)
+    sp = KernelSpec(KernelKey(dtype, "rowT", 8, 16, 16, 0, 1))
+    A, Q, Cc = 256, 2, 16
+    x = rnd((1, Cc, Q, A), 7)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.thread_bs, ka.tb_gap = Q * Cc // 16, 1, 4
+    ka.logQ, ka.logC, ka.logN = 1, 4, 13
+    y = simlib.run_sim(sp, x, x.size, ka, ka.ntiles, simlib.twiddle_table(A, dtype)).reshape(1, A, Q, Cc)
+    ref = np.transpose(np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=3), (0, 3, 2, 1))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)
+
+
+PF = [("row1", "float2", 10, 1, 16, 0), ("row1", "double2", 7, 8, 8, 0), ("row1", "float2", 12, 1, 16, 1)]
+
+
+@pytest.mark.parametrize("kind,dtype,logNi,BS,n,split", PF)
+@pytest.mark.parametrize("tbs", [1, 4])
+def test_prefetch_row1(kind, dtype, logNi, BS, n, split, tbs):
+    sp = KernelSpec(KernelKey(dtype, kind, logNi, BS, n, 0, split, 1))
+    N = 1 << logNi
+    bs = BS * 9 + BS // 2
+    x = rnd((bs, N), logNi + 70)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = (bs + BS - 1) // BS, bs, tbs, 3
+    grid = (ka.ntiles + tbs - 1) // tbs
+    y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype)).reshape(bs, N)
+    assert O.rel_l2(y, O.fft_ref(x.astype(simlib.ctype_of(dtype)))) < O.tolerance(dtype, logNi)
+
+
+def test_prefetch_col_and_rowT():
+    dtype = "float2"
+    sp = KernelSpec(KernelKey(dtype, "col", 8, 16, 16, 0, 0, 1))
+    Ni, ncols, outer, log_ncols = 256, 64, 3, 6
+    x = rnd((outer, Ni, ncols), 5)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.thread_bs, ka.tb_gap, ka.log_ncols = outer * ncols // 16, 5, 2, log_ncols
+    lo_bits, hi, lo = simlib.split_tables(8 + log_ncols, dtype)
+    ka.tw_lo_bits = lo_bits
+    y = simlib.run_sim(sp, x, x.size, ka, (ka.ntiles + 4) // 5, simlib.twiddle_table(Ni, dtype), hi, lo).reshape(outer, Ni, ncols)
+    ref = np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=1)
+    ref = ref * np.exp(-2j * np.pi * ((np.arange(Ni)[:, None] * np.arange(ncols)[None, :]) % (Ni * ncols)) / (Ni * ncols))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)
+    sp = KernelSpec(KernelKey(dtype, "rowT", 8, 16, 16, 0, 0, 1))
+    A, Q, Cc = 256, 2, 32
+    x = rnd((2, Cc, Q, A), 7)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.thread_bs, ka.tb_gap = 2 * Q * Cc // 16, 3, 2
+    ka.logQ, ka.logC, ka.logN = 1, 5, 14
+    y = simlib.run_sim(sp, x, x.size, ka, (ka.ntiles + 2) // 3, simlib.twiddle_table(A, dtype)).reshape(2, A, Q, Cc)
+    ref = np.transpose(np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=3), (0, 3, 2, 1))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)

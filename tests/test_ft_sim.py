@@ -18,8 +18,8 @@ def rnd(shape, seed):
 
 
 def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0,
-           inj_m=0, mag=100.0, seed=0):
-    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 1))
+           inj_m=0, mag=100.0, seed=0, split=0, pf=0):
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 1, split, pf))
     N = 1 << logNi
     bs = ntiles * BS
     x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
@@ -99,3 +99,18 @@ def test_injection_on_arbitrary_element_matches_model_delta():
     k = np.arange(128)
     err = (y - O.fft_ref(x)).reshape(4, 8, 128)[2, 5]
     assert np.allclose(err, 50.0 * np.exp(-2j * np.pi * 3 * k / 128), atol=1e-9)
+
+
+def test_ft_with_split_exchange():
+    sp, x, y, c, fl = run_ft("double2", 8, 4, 16, 24, 4, 3, inj_mode=1, correct=1, split=1)
+    assert c[1] == 6 == c[2]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 8)
+
+
+def test_ft_with_prefetch_recomputes_the_located_tile():
+    sp, x, y, c, fl = run_ft("float2", 8, 4, 16, 24, 4, 3, inj_mode=1, correct=1, pf=1)
+    assert c[1] == 6 == c[2]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("float2", 8)
+    sp, x, y, c, fl = run_ft("double2", 10, 1, 8, 20, 5, 2, inj_mode=2, correct=1, inj_every=1000, inj_tile=13, pf=1)
+    assert c[1] == 1 and c[2] == 1 and fl == [(0, 13)]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 10)

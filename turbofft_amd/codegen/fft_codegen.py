@@ -92,6 +92,9 @@ class KernelSpec:
         self.n = k.n
         self.kind = k.kind
         self.ft = bool(k.ft)
+        self.split = bool(k.split)
+        self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
+        self.lds_esize = self.esize // 2 if self.split else self.esize   # bytes per LDS access
         self.passes = radix_passes(self.Ni, self.n)
         self.npass = len(self.passes)
         self.Tr = self.Ni // self.n              # threads per sub-FFT
@@ -120,7 +123,7 @@ class KernelSpec:
             else:
                 self.pads.append(lds_model.choose_padding(self, x))
         self.lds_elems = max([self.phys_const(self.E - 1, p) + 1 for p in self.pads] + [1])
-        self.red_off_bytes = (self.lds_elems * self.esize + 15) // 16 * 16
+        self.red_off_bytes = (self.lds_elems * self.lds_esize + 15) // 16 * 16
         self.lds_bytes = self.red_off_bytes + (3 * (self.threads // WAVE) * 8 if self.ft else 0)
 
     # ---- address helpers (python side) ----
@@ -287,8 +290,9 @@ class KernelEmitter:
             c.ind -= 1
             c("}")
 
-    def emit_lds_write(self, c: Code, q: int):
-        """Store the outputs of pass q in the layout pass q+1 reads."""
+    def emit_lds_write(self, c: Code, q: int, part: str = ""):
+        """Store the outputs of pass q in the layout pass q+1 reads
+        (part = ".x" / ".y" for one round of a split exchange)."""
         sp = self.s
         R = sp.passes[q]
         U = sp.n // R
@@ -310,11 +314,11 @@ class KernelEmitter:
                 step = P * sp.BS
             for o in range(R):
                 reg = u + U * bitrev(o, lR)
-                c(f"LST({self.lds_index(f'a0 + {step * o}u', pad)}, r[{reg}]);")
+                c(f"LST({self.lds_index(f'a0 + {step * o}u', pad)}, r[{reg}]{part});")
             c.ind -= 1
             c("}")
 
-    def emit_lds_read(self, c: Code, q: int):
+    def emit_lds_read(self, c: Code, q: int, part: str = ""):
         sp = self.s
         pad = sp.pads[q - 1]
         if sp.maps[q] == "major":
@@ -324,59 +328,62 @@ class KernelEmitter:
             c("const unsigned b0 = tx;")
             step = sp.threads
         for e in range(sp.n):
-            c(f"r[{e}] = LLD({self.lds_index(f'b0 + {step * e}u', pad)});")
+            c(f"r[{e}]{part} = LLD({self.lds_index(f'b0 + {step * e}u', pad)});")
 
     # ---------- global addressing ----------
-    def emit_tile_decode(self, c: Code):
+    def emit_tile_decode(self, c: Code, tile: str = "tile", sfx: str = ""):
         """Wave-uniform part of the tile's addresses (64-bit, lives in SGPRs)."""
         sp = self.s
         lBS = ilog2(sp.BS)
         lNi = ilog2(sp.Ni)
         if sp.kind == "row1":
-            c(f"const long long row0 = tile << {lBS};")
-            c(f"const long long ubase = row0 << {lNi};")
+            c(f"const long long row0{sfx} = ({tile}) << {lBS};")
+            c(f"const long long ubase{sfx} = row0{sfx} << {lNi};")
         elif sp.kind == "col":
-            c(f"const unsigned tpl = (unsigned)a.log_ncols - {lBS}u;")
-            c("const unsigned ct = (unsigned)(tile & ((1ll << tpl) - 1));")
-            c("const long long outer = tile >> tpl;")
-            c(f"const long long ubase = (outer << ({lNi} + a.log_ncols)) + ((long long)ct << {lBS});")
-            c(f"const long long gstep = {sp.Tr}ll << a.log_ncols;")
+            c(f"const unsigned tpl{sfx} = (unsigned)a.log_ncols - {lBS}u;")
+            c(f"const unsigned ct{sfx} = (unsigned)(({tile}) & ((1ll << tpl{sfx}) - 1));")
+            c(f"const long long outer{sfx} = ({tile}) >> tpl{sfx};")
+            c(f"const long long ubase{sfx} = (outer{sfx} << ({lNi} + a.log_ncols)) + ((long long)ct{sfx} << {lBS});")
+            c(f"const long long gstep{sfx} = {sp.Tr}ll << a.log_ncols;")
         else:
-            c(f"const unsigned ctl = (unsigned)a.logC - {lBS}u;")
-            c("const unsigned ct = (unsigned)(tile & ((1ll << ctl) - 1));")
-            c("const unsigned qd = (unsigned)((tile >> ctl) & ((1ll << a.logQ) - 1));")
-            c("const long long tb = (tile >> (ctl + a.logQ)) << a.logN;")
-            c(f"const long long ubase_in = tb + ((long long)(qd + ((ct << {lBS}) << a.logQ)) << {lNi});")
-            c(f"const unsigned ls = (unsigned)a.logN - {lNi}u;")
-            c(f"const long long ubase_out = tb + (ct << {lBS}) + ((long long)qd << a.logC);")
-            c(f"const long long gstep = {sp.Tr}ll << ls;")
+            c(f"const unsigned ctl{sfx} = (unsigned)a.logC - {lBS}u;")
+            c(f"const unsigned ct{sfx} = (unsigned)(({tile}) & ((1ll << ctl{sfx}) - 1));")
+            c(f"const unsigned qd{sfx} = (unsigned)((({tile}) >> ctl{sfx}) & ((1ll << a.logQ) - 1));")
+            c(f"const long long tb{sfx} = (({tile}) >> (ctl{sfx} + a.logQ)) << a.logN;")
+            c(f"const long long ubase_in{sfx} = tb{sfx} + ((long long)(qd{sfx} + ((ct{sfx} << {lBS}) << a.logQ)) << {lNi});")
+            c(f"const unsigned ls{sfx} = (unsigned)a.logN - {lNi}u;")
+            c(f"const long long ubase_out{sfx} = tb{sfx} + (ct{sfx} << {lBS}) + ((long long)qd{sfx} << a.logC);")
+            c(f"const long long gstep{sfx} = {sp.Tr}ll << ls{sfx};")
+        names = {"row1": ["row0", "ubase"], "col": ["tpl", "ct", "outer", "ubase", "gstep"],
+                 "rowT": ["ctl", "ct", "qd", "tb", "ubase_in", "ls", "ubase_out", "gstep"]}[sp.kind]
+        c(" ".join(f"(void){n}{sfx};" for n in names))
 
-    def emit_load(self, c: Code):
+    def emit_load(self, c: Code, dst: str = "r", sfx: str = ""):
         sp = self.s
         lNi = ilog2(sp.Ni)
         if sp.kind == "row1":
-            c(f"const unsigned gi = (s << {lNi}) + x;")
+            c(f"const unsigned gi{sfx} = (s << {lNi}) + x;")
             if sp.BS > 1:
-                c("if ((row0 + s) < a.nrows) {")
+                c(f"if ((row0{sfx} + s) < a.nrows) {{")
                 c.ind += 1
             for e in range(sp.n):
-                c(f"r[{e}] = GLDU(in, ubase + {sp.Tr * e}, gi);")
+                c(f"{dst}[{e}] = GLDU(in, ubase{sfx} + {sp.Tr * e}, gi{sfx});")
             if sp.BS > 1:
                 c.ind -= 1
                 c("} else {")
                 c.ind += 1
                 for e in range(sp.n):
-                    c(f"r[{e}] = czero(r[0]);")
+                    c(f"{dst}[{e}] = czero({dst}[0]);")
                 c.ind -= 1
                 c("}")
         elif sp.kind == "col":
-            c("const unsigned gi = s + (x << a.log_ncols);")
+            c(f"const unsigned gi{sfx} = s + (x << a.log_ncols);")
             for e in range(sp.n):
-                c(f"r[{e}] = GLDU(in, ubase + {e} * gstep, gi);")
+                c(f"{dst}[{e}] = GLDU(in, ubase{sfx} + {e} * gstep{sfx}, gi{sfx});")
         else:
-            c(f"const unsigned gi = ((s << a.logQ) << {lNi}) + x;")
+            c(f"const unsigned gi{sfx} = ((s << a.logQ) << {lNi}) + x;")
             for e in range(sp.n):
-                c(f"r[{e}] = GLDU(in, ubase_in + {sp.Tr * e}, gi);")
+                c(f"{dst}[{e}] = GLDU(in, ubase_in{sfx} + {sp.Tr * e}, gi{sfx});")
 
     def out_reg(self, e: int) -> int:
         """Register that holds output k = x + Tr*e after the last pass."""
@@ -481,6 +488,12 @@ class KernelEmitter:
 
     # ---------- phases ----------
     def phases(self) -> List[str]:
+        """Barrier-separated phases of one tile.  A complex exchange is
+        [compute, write] | [read, compute ...]; a split exchange is
+        [compute] | [write re] | [read re] | [write im] | [read im, compute ...]:
+        the new real parts land in the .x registers whose old contents have
+        all been written, while the .y registers still hold the old imaginary
+        parts, so no extra registers are needed."""
         sp = self.s
         out: List[str] = []
         for q in range(sp.npass):
@@ -488,11 +501,25 @@ class KernelEmitter:
             self.map_vars(c, q)
             c(f"{self.T2} t;")
             if q == 0:
-                self.emit_load(c)
-                if sp.ft:
-                    self.emit_ft_input(c)
+                if sp.pf:
+                    # this tile's elements were fetched during the previous tile; start the
+                    # fetch of the next one now so it overlaps every pass of this tile
+                    for e in range(sp.n):
+                        c(f"r[{e}] = rn[{e}];")
+                    if sp.ft:
+                        self.emit_ft_input(c)
+                    c("if (has_next) {")
+                    c.ind += 1
+                    self.emit_tile_decode(c, "tile_n", "_n")
+                    self.emit_load(c, "rn", "_n")
+                    c.ind -= 1
+                    c("}")
+                else:
+                    self.emit_load(c)
+                    if sp.ft:
+                        self.emit_ft_input(c)
             else:
-                self.emit_lds_read(c, q)
+                self.emit_lds_read(c, q, ".y" if sp.split else "")
             self.emit_pass_compute(c, q)
             if q == sp.npass - 1:
                 if sp.ft:
@@ -503,10 +530,24 @@ class KernelEmitter:
             else:
                 c("(void)t;")
                 out.append(c.text())
-                w = Code()
-                self.map_vars(w, q)
-                self.emit_lds_write(w, q)
-                out.append(w.text())
+                if not sp.split:
+                    w = Code()
+                    self.map_vars(w, q)
+                    self.emit_lds_write(w, q)
+                    out.append(w.text())
+                else:
+                    w = Code()
+                    self.map_vars(w, q)
+                    self.emit_lds_write(w, q, ".x")
+                    out.append(w.text())
+                    rd = Code()
+                    self.map_vars(rd, q + 1)
+                    self.emit_lds_read(rd, q + 1, ".x")
+                    out.append(rd.text())
+                    w = Code()
+                    self.map_vars(w, q)
+                    self.emit_lds_write(w, q, ".y")
+                    out.append(w.text())
         return out
 
     # ---------- whole kernel ----------
@@ -515,7 +556,7 @@ class KernelEmitter:
         c = Code()
         T2, R = self.T2, self.R
         c(f"// {sp.name}: {sp.kind} kernel, {T2}, Ni={sp.Ni}, BS={sp.BS}, n={sp.n}, passes={'x'.join(map(str, sp.passes))},")
-        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
+        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
         if sim:
             c(f'extern "C" void {sp.name}_sim(const {T2}* in, {T2}* out, const {T2}* tw, const tfft_kargs* ap, long long grid, const long long* limits)')
             c("{")
@@ -525,11 +566,12 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx;")
-            c(f"std::vector<{T2}> ldsv({sp.lds_elems}); {T2}* lds = ldsv.data();")
+            LT = R if sp.split else T2
+            c(f"std::vector<{LT}> ldsv({sp.lds_elems}); {LT}* lds = ldsv.data();")
             c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
         else:
             c(f'extern "C" __global__ __launch_bounds__({sp.threads})')
@@ -537,11 +579,14 @@ class KernelEmitter:
             c("{")
             c.ind += 1
             c("extern __shared__ __align__(16) unsigned char lds_raw[];")
-            c(f"{T2}* lds = ({T2}*)lds_raw;")
+            LT = R if sp.split else T2
+            c(f"{LT}* lds = ({LT}*)lds_raw;")
             c("const unsigned tx = threadIdx.x;")
             c("const long long grid = gridDim.x;")
             c("long long bx = blockIdx.x;")
             c(f"{T2} r[{sp.n}];")
+            if sp.pf:
+                c(f"{T2} rn[{sp.n}];")
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
         # XCD-aware renumbering: hardware deals blocks round-robin to the 8 XCDs, so block
@@ -559,6 +604,16 @@ class KernelEmitter:
         c("const long long tile0 = chunk * a.tb_gap * a.thread_bs + bx % a.tb_gap;")
         c("int count = 0;")
         c("if (tile0 < a.ntiles) { const long long left = (a.ntiles - tile0 + gstride - 1) / gstride; count = left < a.thread_bs ? (int)left : a.thread_bs; }")
+        if sp.pf:
+            c("if (count > 0) {")
+            c.ind += 1
+            self.emit_tile_decode(c, "tile0", "_n")
+            pre = Code()
+            self.map_vars(pre, 0)
+            self.emit_load(pre, "rn", "_n")
+            self.thread_block(c, sim, pre.text())
+            c.ind -= 1
+            c("}")
         if sp.ft:
             c("long long redo_tile = -1; int extra = 0;")
             c("for (int it = 0; it < count + extra; ++it) {")
@@ -574,6 +629,10 @@ class KernelEmitter:
             c("for (int it = 0; it < count; ++it) {")
             c.ind += 1
             c("const long long tile = tile0 + it * gstride;")
+        if sp.pf:
+            c("const bool has_next = it + 1 < count;")
+            c("const long long tile_n = tile0 + (long long)(it + 1) * gstride;")
+            c("(void)has_next; (void)tile_n;")
         self.emit_tile_decode(c)
         phases = self.phases()
         for i, ph in enumerate(phases):
@@ -582,19 +641,20 @@ class KernelEmitter:
                     c("// ---- barrier ----")
                 else:
                     c("__syncthreads();")
-            if sim:
-                c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
-                c.ind += 1
-                c("auto& r = ts[tx].r; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
-                c("(void)fin1; (void)fin2; (void)fo1; (void)fo2;")
-            else:
-                c("{")
-                c.ind += 1
-            c(ph.rstrip("\n"))
-            c.ind -= 1
-            c("}")
+            self.thread_block(c, sim, ph)
         if sp.ft:
             self.emit_ft_decide(c, sim)
+            if sp.pf:
+                # the tile to recompute is known only now: fetch it for the extra trip
+                c("if (extra && it == count - 1) {")
+                c.ind += 1
+                self.emit_tile_decode(c, "redo_tile", "_n")
+                pre = Code()
+                self.map_vars(pre, 0)
+                self.emit_load(pre, "rn", "_n")
+                self.thread_block(c, sim, pre.text())
+                c.ind -= 1
+                c("}")
         c.ind -= 1
         c("}")  # tile loop
         if sim:
@@ -603,6 +663,22 @@ class KernelEmitter:
         c.ind -= 1
         c("}")
         return c.text()
+
+    def thread_block(self, c: Code, sim: bool, body: str):
+        """Per-thread code: a plain block on the GPU, a loop over the block's
+        threads in the CPU lock-step flavour."""
+        sp = self.s
+        if sim:
+            c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
+            c.ind += 1
+            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
+            c("(void)r; (void)rn; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+        else:
+            c("{")
+            c.ind += 1
+        c(body.rstrip("\n"))
+        c.ind -= 1
+        c("}")
 
     def emit_ft_decide(self, c: Code, sim: bool):
         """Block-wide reduction and the detect / locate decision
@@ -683,7 +759,7 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     kinds = {"row1": 0, "col": 1, "rowT": 2}
     for sp in specs:
         k = sp.key
-        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {sp.threads}, {sp.lds_bytes}}},')
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {sp.threads}, {sp.lds_bytes}}},')
     c("};")
     c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")

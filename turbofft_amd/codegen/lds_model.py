@@ -43,10 +43,10 @@ def exchange_write_cost(spec, x: int, pad: Tuple[int, int]) -> Tuple[int, int]:
     for w in waves:
         for u in range(U):
             for o in range(R):
-                addrs = [spec.phys_const(spec.logical_write_addr(x, w * 64 + lane, u, o), pad) * spec.esize
+                addrs = [spec.phys_const(spec.logical_write_addr(x, w * 64 + lane, u, o), pad) * spec.lds_esize
                          for lane in range(64)]
-                total += access_cost(addrs, spec.esize)
-                ideal += max(1, 64 * spec.esize // (BANKS * BANK_BYTES))
+                total += access_cost(addrs, spec.lds_esize)
+                ideal += max(1, 64 * spec.lds_esize // (BANKS * BANK_BYTES))
     return total, ideal
 
 
@@ -54,9 +54,9 @@ def exchange_read_cost(spec, x: int, pad: Tuple[int, int]) -> Tuple[int, int]:
     total = 0
     ideal = 0
     for e in range(spec.n):
-        addrs = [spec.phys_const(spec.logical_read_addr(x + 1, lane, e), pad) * spec.esize for lane in range(64)]
-        total += access_cost(addrs, spec.esize)
-        ideal += max(1, 64 * spec.esize // (BANKS * BANK_BYTES))
+        addrs = [spec.phys_const(spec.logical_read_addr(x + 1, lane, e), pad) * spec.lds_esize for lane in range(64)]
+        total += access_cost(addrs, spec.lds_esize)
+        ideal += max(1, 64 * spec.lds_esize // (BANKS * BANK_BYTES))
     return total, ideal
 
 

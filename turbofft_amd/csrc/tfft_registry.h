@@ -11,6 +11,8 @@ typedef struct tfft_kernel_entry {
     int datatype;        // 0 = float2, 1 = double2
     int kind;            // 0 = row1, 1 = col, 2 = rowT
     int logNi, BS, n, ft;
+    int split;           // 1: re and im are exchanged through LDS in two rounds
+    int pf;              // 1: the block prefetches its next tile (wants a persistent grid)
     int threads;         // block size
     int lds_bytes;       // dynamic LDS
 } tfft_kernel_entry;

@@ -47,7 +47,9 @@ constexpr double kPi = 3.14159265358979323846;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[11];
+    int v[17];           // 11 reference columns + optional per-launch flags: split exchange, prefetch
+    int split(int i) const { return v[11 + i]; }
+    int pf(int i) const { return v[14 + i]; }
     int logN() const { return v[0]; }
     int launches() const { return v[1]; }
     int logNi(int i) const { return v[2 + i]; }
@@ -66,7 +68,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 11 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 17 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -78,12 +80,12 @@ int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
     return i == launches - 1 ? 2 : 1;
 }
 
-const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft) {
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf) {
     int cnt = 0;
     const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
-            t[i].n == n && t[i].ft == ft)
+            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf)
             return &t[i];
     return nullptr;
 }
@@ -164,6 +166,7 @@ struct turbofft_plan {
     int launches = 0;
     const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
     int tb_gap[3] = {1, 1, 1};
+    int resident[3] = {1, 1, 1};   // blocks of launch i that fit on the device at once
     size_t esize = 8;
     // device tables
     void* tw = nullptr;          // concatenated twiddle table, 2*tw_N - 1 entries
@@ -278,10 +281,10 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     long long twN = 1;
     for (int i = 0; i < p->launches; ++i) {
         int kind = kind_of_launch(p->launches, i);
-        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft);
+        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0);
         if (!k)
-            return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d)",
-                        i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft);
+            return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
+                        i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
         p->k[i] = k;
         if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
             HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
@@ -289,6 +292,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
         HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k->func, k->threads, k->lds_bytes));
         if (nb < 1) return fail(TURBOFFT_ENOPLAN, "kernel %s does not fit on a CU (LDS %d B)", k->name, k->lds_bytes);
         p->tb_gap[i] = nb * prop.multiProcessorCount;      // fft_codegen.py:216-218 with measured residency
+        p->resident[i] = p->tb_gap[i];
         if ((1ll << r.logNi(i)) > twN) twN = 1ll << r.logNi(i);
         if (kind == 1) {
             // inter-launch twiddle W_(2^L)^e, L = log2(Ni * ncols): e = hi << lo_bits | lo
@@ -498,6 +502,12 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         a.nrows = bs;
         a.thread_bs = p->thread_bs;
         a.tb_gap = p->tb_gap[i];
+        if (k->pf && !p->if_ft && p->thread_bs == 1 && a.ntiles > p->resident[i]) {
+            // prefetching kernels run as a persistent grid: one block per resident slot walks
+            // the tiles with the grid as stride, so there is always a next tile to fetch
+            a.tb_gap = p->resident[i];
+            a.thread_bs = (int)((a.ntiles + p->resident[i] - 1) / p->resident[i]);
+        }
         a.xcd_chunk = p->xcd_chunk;
         int kind = kind_of_launch(p->launches, i);
         if (kind == 1) {
@@ -531,7 +541,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.ft.err_smoothing = p->err_smoothing;
             a.ft.err_threshold = p->err_threshold;
         }
-        long long grid = (a.ntiles + p->thread_bs - 1) / p->thread_bs;
+        long long grid = (a.ntiles + a.thread_bs - 1) / a.thread_bs;
         if (grid < 1) continue;
         if (grid > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "grid of %lld blocks exceeds the launch limit", grid);
         const void* in_arg = src[i];
