@@ -15,8 +15,13 @@ extern "C" {
 #endif
 
 typedef struct tfft_ft_args {
-    const void* cksum;            /* c_Ni, Ni entries of T (input-side encoding vector)   */
-    unsigned long long* counters; /* [0]=groups checked [1]=detected [2]=corrected
+    const void* cksum;            /* Ni entries of T: (re c + im c, re c - im c) of the input-
+                                     side encoding vector c_Ni, so that re+im of x*c costs two
+                                     fused multiply-adds                                      */
+    unsigned long long* counters; /* [4]=detections (also the next free slot of `flagged`),
+                                     [3]=detections whose located tile was out of range;
+                                     groups checked are counted on the host and corrected =
+                                     detected - uncorrectable while `correct` is set; [0..2] unused
                                      [3]=uncorrectable  [4]=flagged-list length            */
     long long* flagged;           /* flagged tile ids: flagged[2*i]=launch, [2*i+1]=tile   */
     int flagged_cap;

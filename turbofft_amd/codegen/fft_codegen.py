@@ -445,13 +445,15 @@ class KernelEmitter:
     # ---------- fault tolerance ----------
     def emit_ft_input(self, c: Code):
         """in1 += re+im of x*c[m]; in2 += cnt * (...)   (fft_codegen.py:354-367),
-        then the optional compute-side error injection (:412-415)."""
+        then the optional compute-side error injection (:412-415).
+        re+im of x*c = x.re*(c.re+c.im) + x.im*(c.re-c.im): the table holds the two
+        real factors, so an element costs two fused multiply-adds."""
         sp = self.s
         c("if (!is_redo) {")
         c.ind += 1
         c(f"{self.R} acc = 0;")
         for e in range(sp.n):
-            c(f"{{ const {self.T2} cv = TWLD(ck, x + {sp.Tr * e}u); const {self.T2} p = cmul(r[{e}], cv); acc += p.x + p.y; }}")
+            c(f"{{ const {self.T2} cv = TWLD(ck, x + {sp.Tr * e}u); acc += r[{e}].x * cv.x + r[{e}].y * cv.y; }}")
         c("fin1 += acc; fin2 += cntf * acc;")
         c("if (inj_hit && s == (unsigned)a.ft.inj_s && x == ((unsigned)a.ft.inj_m & %du)) {" % (sp.Tr - 1))
         c.ind += 1
@@ -465,23 +467,24 @@ class KernelEmitter:
 
     def emit_ft_output(self, c: Code):
         """out1 -= re+im of y*r[k%3]; out2 -= cnt * (...)   (fft_codegen.py:374-384),
-        taken before the inter-launch twiddle."""
+        taken before the inter-launch twiddle.  re+im of y*r = y.re*(r.re+r.im) +
+        y.im*(r.re-r.im); the three (sum, difference) pairs are rotated by x % 3 once."""
         sp = self.s
         c("if (!is_redo) {")
         c.ind += 1
         c("const unsigned x3 = x % 3u;")
-        s3 = self.lit(0.8660253882408142)
-        c(f"const {self.R} rrx0 = (x3 == 0u) ? ({self.R})1 : ({self.R})-0.5;")
-        c(f"const {self.R} rry0 = (x3 == 0u) ? ({self.R})0 : ((x3 == 1u) ? -{s3} : {s3});")
-        c(f"const {self.R} rrx1 = (x3 == 2u) ? ({self.R})1 : ({self.R})-0.5;")
-        c(f"const {self.R} rry1 = (x3 == 2u) ? ({self.R})0 : ((x3 == 0u) ? -{s3} : {s3});")
-        c(f"const {self.R} rrx2 = (x3 == 1u) ? ({self.R})1 : ({self.R})-0.5;")
-        c(f"const {self.R} rry2 = (x3 == 1u) ? ({self.R})0 : ((x3 == 2u) ? -{s3} : {s3});")
+        s3 = 0.8660253882408142
+        pq = [(1.0, 1.0), (-0.5 - s3, -0.5 + s3), (-0.5 + s3, -0.5 - s3)]      # r[0], r[1], r[2]
+        for cc in range(3):
+            # element class cc uses r[(x3 + cc) % 3]
+            sel = [pq[(v + cc) % 3] for v in range(3)]
+            c(f"const {self.R} rp{cc} = (x3 == 0u) ? {self.lit(sel[0][0])} : ((x3 == 1u) ? {self.lit(sel[1][0])} : {self.lit(sel[2][0])});")
+            c(f"const {self.R} rq{cc} = (x3 == 0u) ? {self.lit(sel[0][1])} : ((x3 == 1u) ? {self.lit(sel[1][1])} : {self.lit(sel[2][1])});")
         c(f"{self.R} acc = 0;")
         for e in range(sp.n):
             ce = (sp.Tr * e) % 3
             reg = self.out_reg(e)
-            c(f"{{ const {self.T2} p = cmulc(r[{reg}], rrx{ce}, rry{ce}); acc += p.x + p.y; }}")
+            c(f"acc += r[{reg}].x * rp{ce} + r[{reg}].y * rq{ce};")
         c("fo1 -= acc; fo2 -= cntf * acc;")
         c.ind -= 1
         c("}")
@@ -592,18 +595,24 @@ class KernelEmitter:
         # XCD-aware renumbering: hardware deals blocks round-robin to the 8 XCDs, so block
         # b runs on XCD b % 8.  Give every XCD chunks of `xcd_chunk` consecutive tiles (its
         # L2 then streams contiguous memory) while the 8 XCDs stay in one neighbourhood.
+        # (block and tile counts fit 32 bits: the host rejects larger grids)
         c("if (a.xcd_chunk > 0) {")
-        c("    const long long span = 8ll * a.xcd_chunk, full = (grid / span) * span;")
-        c("    if (bx < full) { const long long q = bx >> 3, xcd = bx & 7; bx = (q / a.xcd_chunk) * span + xcd * a.xcd_chunk + q % a.xcd_chunk; }")
+        c("    const unsigned ub = (unsigned)bx, xc = (unsigned)a.xcd_chunk, span = 8u * xc, full = ((unsigned)grid / span) * span;")
+        c("    if (ub < full) { const unsigned q = ub >> 3, xcd = ub & 7u; bx = (long long)((q / xc) * span + xcd * xc + q % xc); }")
         c("}")
         c(f"const {T2}* twhi = (const {T2}*)a.tw_hi; const {T2}* twlo = (const {T2}*)a.tw_lo; const {T2}* ck = (const {T2}*)a.ft.cksum;")
         c("(void)twhi; (void)twlo; (void)ck;")
         # tile group of this block (fft_codegen.py:218,260-261 with a rounded-up grid)
-        c("const long long chunk = bx / a.tb_gap;")
-        c("const long long gstride = ((chunk + 1) * a.tb_gap <= grid) ? a.tb_gap : (grid - chunk * a.tb_gap);")
-        c("const long long tile0 = chunk * a.tb_gap * a.thread_bs + bx % a.tb_gap;")
-        c("int count = 0;")
-        c("if (tile0 < a.ntiles) { const long long left = (a.ntiles - tile0 + gstride - 1) / gstride; count = left < a.thread_bs ? (int)left : a.thread_bs; }")
+        c("long long gstride = 1, tile0 = bx;")
+        c("int count = bx < a.ntiles ? 1 : 0;")
+        c("if (a.thread_bs > 1) {")
+        c("    const unsigned ub = (unsigned)bx, gap = (unsigned)a.tb_gap, ug = (unsigned)grid, tbs = (unsigned)a.thread_bs;")
+        c("    const unsigned chunk = ub / gap;")
+        c("    const unsigned gs = ((chunk + 1u) * gap <= ug) ? gap : (ug - chunk * gap);")
+        c("    const unsigned long long t0 = (unsigned long long)chunk * gap * tbs + ub % gap;")
+        c("    gstride = gs; tile0 = (long long)t0; count = 0;")
+        c("    if (tile0 < a.ntiles) { const unsigned left = (unsigned)((a.ntiles - tile0 + gs - 1) / gs); count = left < tbs ? (int)left : (int)tbs; }")
+        c("}")
         if sp.pf:
             c("if (count > 0) {")
             c.ind += 1
@@ -708,21 +717,17 @@ class KernelEmitter:
         c("if (tx == 0) {")
         c.ind += 1
         if sim:
-            c("a.ft.counters[0] += 1;")
             c("if (det) {")
-            c("    a.ft.counters[1] += 1;")
             c("    const unsigned long long slot = a.ft.counters[4]++;")
             c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
-            c("    if (valid && a.ft.correct) a.ft.counters[2] += 1;")
             c("    if (!valid) a.ft.counters[3] += 1;")
             c("}")
         else:
-            c("atomicAdd(&a.ft.counters[0], 1ull);")
+            # one atomic per detection: the slot counter is also the detection count, and
+            # corrected = detected - uncorrectable when correction is on
             c("if (det) {")
-            c("    atomicAdd(&a.ft.counters[1], 1ull);")
             c("    const unsigned long long slot = atomicAdd(&a.ft.counters[4], 1ull);")
             c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
-            c("    if (valid && a.ft.correct) atomicAdd(&a.ft.counters[2], 1ull);")
             c("    if (!valid) atomicAdd(&a.ft.counters[3], 1ull);")
             c("}")
         c.ind -= 1

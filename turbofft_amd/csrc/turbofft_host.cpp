@@ -185,6 +185,7 @@ struct turbofft_plan {
     double inj_mag = 100.0;
     int cksum_mode = 0;
     int xcd_chunk = 64;          // tiles per XCD chunk (0 = plain block order)
+    unsigned long long checked = 0;   // checksum groups launched since the last reset
 };
 
 extern "C" {
@@ -341,6 +342,11 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             std::vector<char> host((size_t)Ni * p->esize);
             int rc = turbofft_build_checksum_vector(p->datatype, Ni, p->cksum_mode, host.data());
             if (rc) return rc;
+            // device form: (re c + im c, re c - im c)
+            for (long long m = 0; m < Ni; ++m) {
+                if (p->datatype == TURBOFFT_FP32) { c32& v = ((c32*)host.data())[m]; float a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
+                else { c64& v = ((c64*)host.data())[m]; double a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
+            }
             HIP_TRY(hipMalloc(&p->cksum[i], host.size()));
             HIP_TRY(hipMemcpy(p->cksum[i], host.data(), host.size(), hipMemcpyHostToDevice));
         }
@@ -444,6 +450,7 @@ int turbofft_set_injection(turbofft_plan_t* p, int mode, int launch, int every, 
 
 int turbofft_reset_ft_counters(turbofft_plan_t* p) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    p->checked = 0;
     if (!p->if_ft) return TURBOFFT_OK;
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemset(p->counters, 0, 8 * sizeof(unsigned long long)));
@@ -460,9 +467,11 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
         HIP_TRY(hipDeviceSynchronize());
         HIP_TRY(hipMemcpy(c, p->counters, sizeof c, hipMemcpyDeviceToHost));
     }
-    if (checked) *checked = c[0];
-    if (detected) *detected = c[1];
-    if (corrected) *corrected = c[2];
+    if (checked) *checked = p->checked;
+    // one device counter per event class: [4] detections, [3] detections that could not be
+    // located; every located detection is recomputed while correction is switched on
+    if (detected) *detected = c[4];
+    if (corrected) *corrected = p->correct ? c[4] - c[3] : 0;
     if (uncorrectable) *uncorrectable = c[3];
     int n = (int)(c[4] < (unsigned long long)p->flagged_cap ? c[4] : (unsigned long long)p->flagged_cap);
     if (n > cap) n = cap < 0 ? 0 : cap;
@@ -544,6 +553,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         long long grid = (a.ntiles + a.thread_bs - 1) / a.thread_bs;
         if (grid < 1) continue;
         if (grid > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "grid of %lld blocks exceeds the launch limit", grid);
+        if (p->if_ft) p->checked += (unsigned long long)grid;   // one checksum group per block
         const void* in_arg = src[i];
         void* out_arg = dst[i];
         const void* tw_arg = p->tw;
