@@ -183,3 +183,23 @@ def test_prefetch_col_and_rowT():
     y = simlib.run_sim(sp, x, x.size, ka, (ka.ntiles + 2) // 3, simlib.twiddle_table(A, dtype)).reshape(2, A, Q, Cc)
     ref = np.transpose(np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=3), (0, 3, 2, 1))
     assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)
+
+
+XL = [("float2", 7, 8, 8), ("double2", 10, 1, 8), ("float2", 8, 4, 8), ("float2", 10, 2, 16), ("float2", 11, 1, 16),
+      ("double2", 11, 2, 8), ("float2", 9, 8, 4)]
+
+
+@pytest.mark.parametrize("dtype,logNi,BS,n", XL)
+def test_cross_lane_last_pass(dtype, logNi, BS, n):
+    # the final radix-2/4/8 pass runs across adjacent lanes (DPP / ds_swizzle on the GPU)
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 0, 0, 0, 1))
+    assert sp.xl and sp.RL in (2, 4, 8) and len(sp.pads) == sp.npass - 2
+    N = 1 << logNi
+    bs = BS * 5 + BS // 2
+    x = rnd((bs, N), logNi + 90)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = (bs + BS - 1) // BS, bs, 2, 3
+    y = simlib.run_sim(sp, x, bs * N, ka, (ka.ntiles + 1) // 2, simlib.twiddle_table(N, dtype)).reshape(bs, N)
+    ref = O.fft_ref(x.astype(simlib.ctype_of(dtype)))
+    for b in range(bs):
+        assert O.rel_l2(y[b], ref[b]) < O.tolerance(dtype, logNi)

@@ -164,3 +164,40 @@ def test_cli_verify_mode():
         assert "Compare begin." in r.stdout and "Compare finished." in r.stdout
         assert "Error detected" not in r.stdout
         assert f"turboFFT, {logN}, " in r.stdout
+
+
+VARIANTS_DIR = os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param", "gfx950")
+
+
+def _variant_rows(dt):
+    from turbofft_amd.codegen.plan import load_plan_csv
+    return [r for r in load_plan_csv(os.path.join(VARIANTS_DIR, f"variants_{dt}.csv")) if r.launches]
+
+
+@pytest.mark.parametrize("dt", ["float2", "double2"])
+def test_optional_kernel_variants(dt):
+    # rows of variants_<T>.csv: split exchange, next-tile prefetch and cross-lane last pass
+    # kernels that the default table does not use; every one must meet the same accuracy bar
+    path = os.path.join(VARIANTS_DIR, f"variants_{dt}.csv")
+    rows = _variant_rows(dt)
+    assert rows
+    for r in rows:
+        plan = turbofft_amd.TurboFFT(r.logN, dt, param_csv=path)
+        BS = plan.BS[0] if plan.launches == 1 else 1
+        bs = 70 * BS + max(1, BS // 2) if r.logN <= 13 else 5      # many tiles: the prefetch loop must iterate
+        x = make(bs, 1 << r.logN, dt, 100 + r.logN)
+        y = gpu_fft(plan, x)
+        ref = O.fft_ref(x)
+        for b in range(bs):
+            assert O.rel_l2(y[b], ref[b]) <= O.tolerance(dt, r.logN), (r, b)
+        # the same rows with fault tolerance (cross-lane rows fall back to the LDS kernel)
+        # (tight detection rule: with the default one the error's own share of the checksum
+        # magnitude keeps the ratio of an 8192-point tile next to the threshold)
+        planf = turbofft_amd.TurboFFT(r.logN, dt, if_err=1, thread_bs=3, param_csv=path)
+        planf.set_ft_params(0.0, 1e-4 if dt == "float2" else 1e-9, correct=True)
+        planf.set_injection(1, mag=1e3)
+        yf = gpu_fft(planf, x)
+        c = planf.ft_counters()
+        assert c["detected"] == c["corrected"] > 0 and c["uncorrectable"] == 0
+        for b in range(bs):
+            assert O.rel_l2(yf[b], ref[b]) <= O.tolerance(dt, r.logN), (r, b, "ft")

@@ -43,9 +43,11 @@ def test_builtin_rows_match_csv_and_are_consistent(dtype):
     assert len(rows) >= 26
     for logN in range(1, 26):
         r = turbofft_amd.builtin_plan_row(dtype, logN)
-        p = P.PlanRow.from_list(r)
-        assert p == rows[logN] and p.logN == logN and sum(p.logNi) == logN
-        for i, k in enumerate(P.kernels_for_row(p, dtype, 0)):
+        p = P.PlanRow.from_list(r)                       # the 11 reference columns
+        full = rows[logN]                                # ... plus this build's optional flags
+        assert (p.logN, p.launches, p.logNi, p.BS, p.n) == (full.logN, full.launches, full.logNi, full.BS, full.n)
+        assert p.logN == logN and sum(p.logNi) == logN
+        for i, k in enumerate(P.kernels_for_row(full, dtype, 0) + P.kernels_for_row(full, dtype, 1)):
             sp = KernelSpec(k)
             assert sp.threads % 64 == 0 and sp.threads <= 1024
             assert sp.lds_bytes <= 160 * 1024

@@ -94,6 +94,7 @@ class KernelSpec:
         self.ft = bool(k.ft)
         self.split = bool(k.split)
         self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
+        self.xl = bool(k.xl)        # last (radix 2/4/8) pass across lanes instead of through LDS
         self.lds_esize = self.esize // 2 if self.split else self.esize   # bytes per LDS access
         self.passes = radix_passes(self.Ni, self.n)
         self.npass = len(self.passes)
@@ -115,9 +116,19 @@ class KernelSpec:
         self.P = [1]
         for R in self.passes:
             self.P.append(self.P[-1] * R)
+        # passes that end with an LDS exchange or the global store; with a cross-lane last
+        # pass the final radix is folded into the pass before it
+        self.npass_lds = self.npass
+        if self.xl:
+            self.RL = self.passes[-1]
+            if (self.kind != "row1" or self.ft or self.npass < 3 or self.RL not in (2, 4, 8)
+                    or self.passes[-2] != self.n or self.Tr % self.RL):
+                raise ValueError(f"{k}: the cross-lane last pass needs a row1 non-FT kernel with >= 3 passes "
+                                 f"ending in radix 2, 4 or 8 (passes {self.passes})")
+            self.npass_lds = self.npass - 1
         # padding per exchange x (between pass x and x+1)
         self.pads: List[Tuple[int, int]] = []
-        for x in range(self.npass - 1):
+        for x in range(self.npass_lds - 1):
             if self.pad_override and x in self.pad_override:
                 self.pads.append(self.pad_override[x])
             else:
@@ -149,8 +160,13 @@ class KernelSpec:
 
     def thread_sx(self, q: int, tx: int) -> Tuple[int, int]:
         if self.maps[q] == "major":
-            return tx // self.Tr, tx % self.Tr
-        return tx % self.BS, tx // self.BS
+            s, x = tx // self.Tr, tx % self.Tr
+        else:
+            s, x = tx % self.BS, tx // self.BS
+        if self.xl and q == self.npass_lds - 1:
+            # partners of the cross-lane pass sit in adjacent lanes: j in the low bits
+            x = (x // self.RL) + (x % self.RL) * self.P[q]
+        return s, x
 
     def layout_addr(self, kind: str, s: int, pos: int) -> int:
         return s * self.Ni + pos if kind == "major" else s + self.BS * pos
@@ -181,10 +197,17 @@ class KernelEmitter:
     # ---------- thread map ----------
     def map_vars(self, c: Code, q: int):
         sp = self.s
+        xn = "x"
+        if sp.xl and q == sp.npass_lds - 1:
+            xn = "xraw"
         if sp.maps[q] == "major":
-            c(f"const unsigned s = tx >> {ilog2(sp.Tr)}, x = tx & {sp.Tr - 1}u;")
+            c(f"const unsigned s = tx >> {ilog2(sp.Tr)}, {xn} = tx & {sp.Tr - 1}u;")
         else:
-            c(f"const unsigned s = tx & {sp.BS - 1}u, x = tx >> {ilog2(sp.BS)};")
+            c(f"const unsigned s = tx & {sp.BS - 1}u, {xn} = tx >> {ilog2(sp.BS)};")
+        if xn == "xraw":
+            # the RL partners of the cross-lane pass are adjacent lanes: sub-index j = xraw % RL,
+            # completed digits low = xraw / RL; x is the row position low + P*j the pass works on
+            c(f"const unsigned x = (xraw >> {ilog2(sp.RL)}) + ((xraw & {sp.RL - 1}u) << {ilog2(sp.P[q])});")
 
     def lds_index(self, expr: str, pad: Tuple[int, int]) -> str:
         ps, pl = pad
@@ -490,16 +513,78 @@ class KernelEmitter:
         c("}")
 
     # ---------- phases ----------
-    def phases(self) -> List[str]:
-        """Barrier-separated phases of one tile.  A complex exchange is
-        [compute, write] | [read, compute ...]; a split exchange is
-        [compute] | [write re] | [read re] | [write im] | [read im, compute ...]:
-        the new real parts land in the .x registers whose old contents have
-        all been written, while the .y registers still hold the old imaginary
-        parts, so no extra registers are needed."""
+    def emit_xlane_pass(self, c: Code, q: int) -> List[str]:
+        """The last radix-RL DFT across RL adjacent lanes, on every register:
+        log2(RL) radix-2 DIF stages, partner = lane ^ half through DPP quad
+        permutes (half 1, 2) or ds_swizzle (half 4).  Lane j ends with output
+        digit bitrev(j).  Returns the phase texts (the lock-step CPU flavour
+        needs a thread-loop boundary before each stage)."""
         sp = self.s
-        out: List[str] = []
-        for q in range(sp.npass):
+        RL, n = sp.RL, sp.n
+        out = []
+        length = RL
+        while length >= 2:
+            half = length // 2
+            st = Code()
+            self.map_vars(st, q)
+            st("(void)x; (void)s;")
+            st(f"// cross-lane stage: span {length}, partner = lane ^ {half}")
+            st("{")
+            st.ind += 1
+            st(f"const unsigned jj = xraw & {length - 1}u;")
+            st(f"const bool hi = (jj & {half}u) != 0u;")
+            st(f"const {self.R} sg = hi ? ({self.R})-1 : ({self.R})1;")
+            if length > 2:
+                # upper lanes multiply by W_length^(jj - half)
+                st(f"{self.R} wr = 1, wi = 0;")
+                for kk in range(1, half):
+                    ang = -2.0 * math.pi * kk / length
+                    st(f"if (jj == {half + kk}u) {{ wr = {self.lit(math.cos(ang))}; wi = {self.lit(math.sin(ang))}; }}")
+            st(f"{self.T2} pv;")
+            for i in range(n):
+                st(f"XLANE({i}, {half}, pv);")
+                st(f"r[{i}].x = pv.x + sg * r[{i}].x; r[{i}].y = pv.y + sg * r[{i}].y;")
+                if length > 2:
+                    st(f"r[{i}] = cmulc(r[{i}], wr, wi);")
+            st.ind -= 1
+            st("}")
+            out.append(st.text())
+            length = half
+        return out
+
+    def emit_store_xlane(self, c: Code, q: int):
+        """Store after the cross-lane pass: register o of lane j holds
+        k = low + P*o + (Ni/RL)*bitrev(j)."""
+        sp = self.s
+        lNi = ilog2(sp.Ni)
+        RL, L = sp.RL, ilog2(sp.RL)
+        P = sp.P[q]
+        lR = ilog2(sp.n)
+        c(f"const unsigned jl = xraw & {RL - 1}u;")
+        brev = {1: "jl", 2: "(((jl & 1u) << 1) | (jl >> 1))", 3: "(((jl & 1u) << 2) | (jl & 2u) | (jl >> 2))"}[L]
+        c(f"const unsigned kb = (xraw >> {L}) + ({brev} << {lNi - L});")
+        c(f"const unsigned go = (s << {lNi}) + kb;")
+        if sp.BS > 1:
+            c("if ((row0 + s) < a.nrows) {")
+            c.ind += 1
+        for o in range(sp.n):
+            c(f"GSTU(out, ubase + {P * o}, go, r[{bitrev(o, lR)}]);")
+        if sp.BS > 1:
+            c.ind -= 1
+            c("}")
+
+    def phases(self) -> List[Tuple[str, str]]:
+        """Phases of one tile as (separator before, text).  Separator "barrier"
+        is a block barrier; "lane" is nothing on the GPU (lanes of a wavefront
+        run in lock step) and a thread-loop boundary in the CPU flavour.
+        A complex exchange is [compute] b [write] b [read, compute ...]; a split
+        exchange is [compute] b [write re] b [read re] b [write im] b [read im,
+        compute ...]: the new real parts land in the .x registers whose old
+        contents have all been written, while the .y registers still hold the
+        old imaginary parts, so no extra registers are needed."""
+        sp = self.s
+        out: List[Tuple[str, str]] = []
+        for q in range(sp.npass_lds):
             c = Code()
             self.map_vars(c, q)
             c(f"{self.T2} t;")
@@ -524,33 +609,49 @@ class KernelEmitter:
             else:
                 self.emit_lds_read(c, q, ".y" if sp.split else "")
             self.emit_pass_compute(c, q)
-            if q == sp.npass - 1:
+            if q == sp.npass_lds - 1:
+                if sp.xl:
+                    c("(void)t;")
+                    stages = self.emit_xlane_pass(c, q)
+                    out.append(("barrier", c.text()))
+                    for i, st in enumerate(stages):
+                        # (the CPU flavour snapshots every thread's registers in a phase of
+                        # its own, so that no thread sees a partner that already moved on)
+                        out.append(("lane", "SNAP();\n"))
+                        if i == len(stages) - 1:
+                            fin = Code()
+                            fin(st.rstrip("\n"))
+                            self.emit_store_xlane(fin, q)
+                            out.append(("lane", fin.text()))
+                        else:
+                            out.append(("lane", st))
+                    continue
                 if sp.ft:
                     self.emit_ft_output(c)
                 self.emit_store(c)
                 c("(void)t;")
-                out.append(c.text())
+                out.append(("barrier", c.text()))
             else:
                 c("(void)t;")
-                out.append(c.text())
+                out.append(("barrier", c.text()))
                 if not sp.split:
                     w = Code()
                     self.map_vars(w, q)
                     self.emit_lds_write(w, q)
-                    out.append(w.text())
+                    out.append(("barrier", w.text()))
                 else:
                     w = Code()
                     self.map_vars(w, q)
                     self.emit_lds_write(w, q, ".x")
-                    out.append(w.text())
+                    out.append(("barrier", w.text()))
                     rd = Code()
                     self.map_vars(rd, q + 1)
                     self.emit_lds_read(rd, q + 1, ".x")
-                    out.append(rd.text())
+                    out.append(("barrier", rd.text()))
                     w = Code()
                     self.map_vars(w, q)
                     self.emit_lds_write(w, q, ".y")
-                    out.append(w.text())
+                    out.append(("barrier", w.text()))
         return out
 
     # ---------- whole kernel ----------
@@ -559,7 +660,7 @@ class KernelEmitter:
         c = Code()
         T2, R = self.T2, self.R
         c(f"// {sp.name}: {sp.kind} kernel, {T2}, Ni={sp.Ni}, BS={sp.BS}, n={sp.n}, passes={'x'.join(map(str, sp.passes))},")
-        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
+        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}{', cross-lane last pass' if sp.xl else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
         if sim:
             c(f'extern "C" void {sp.name}_sim(const {T2}* in, {T2}* out, const {T2}* tw, const tfft_kargs* ap, long long grid, const long long* limits)')
             c("{")
@@ -569,7 +670,7 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx;")
@@ -644,11 +745,11 @@ class KernelEmitter:
             c("(void)has_next; (void)tile_n;")
         self.emit_tile_decode(c)
         phases = self.phases()
-        for i, ph in enumerate(phases):
+        for i, (sep, ph) in enumerate(phases):
             if i:
                 if sim:
-                    c("// ---- barrier ----")
-                else:
+                    c(f"// ---- {sep} ----")
+                elif sep == "barrier":
                     c("__syncthreads();")
             self.thread_block(c, sim, ph)
         if sp.ft:
@@ -764,7 +865,7 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     kinds = {"row1": 0, "col": 1, "rowT": 2}
     for sp in specs:
         k = sp.key
-        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {sp.threads}, {sp.lds_bytes}}},')
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {sp.threads}, {sp.lds_bytes}}},')
     c("};")
     c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")

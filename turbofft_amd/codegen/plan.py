@@ -5,8 +5,8 @@ A plan CSV keeps the reference's 11-column row
 (readme.md:48-60; consumed at fft_codegen.py:745-752 and main.cu:8-9,16,22-24),
 row index == logN.  Three optional trailing columns `x1, x2, x3` select, per
 launch, the split exchange (re and im go through a half-size LDS buffer in two
-rounds), and three more `p1, p2, p3` the next-tile prefetch; a row without them
-means all zeros.  Launch i transforms a digit of size 2^logNi with BSi
+rounds), three more `p1, p2, p3` the next-tile prefetch and three more
+`c1, c2, c3` the cross-lane last pass; a row without them means all zeros.  Launch i transforms a digit of size 2^logNi with BSi
 sub-FFTs per tile and ni elements per thread; launch 0 owns the most-strided
 digit and the last launch the contiguous one.
 """
@@ -25,6 +25,7 @@ class PlanRow:
     n: Tuple[int, ...]
     split: Tuple[int, ...] = ()      # optional columns 12-14: 1 = exchange re and im separately
     pf: Tuple[int, ...] = ()         # optional columns 15-17: 1 = prefetch the next tile
+    xl: Tuple[int, ...] = ()         # optional columns 18-20: 1 = last small-radix pass across lanes
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -36,8 +37,9 @@ class PlanRow:
             raise ValueError(f"launches must be 0..3: {row}")
         ext = (row[11:14] + [0, 0, 0])[:3]
         ext2 = (row[14:17] + [0, 0, 0])[:3]
+        ext3 = (row[17:20] + [0, 0, 0])[:3]
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
-                    tuple(ext2[:L]))
+                    tuple(ext2[:L]), tuple(ext3[:L]))
         if L and sum(p.logNi) != p.logN:
             raise ValueError(f"logN1+logN2+logN3 != logN in row {row}")
         return p
@@ -57,11 +59,12 @@ class KernelKey:
     ft: int
     split: int = 0   # 1: every LDS exchange moves re and im in two rounds through a half-size buffer
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
+    xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
-        return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "")
+        return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
                 + ("_ft" if self.ft else ""))
 
 
@@ -72,7 +75,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:17] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:20] if t.strip()]))
     return rows
 
 
@@ -82,7 +85,10 @@ def launch_kinds(launches: int) -> List[str]:
 
 def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
     return [KernelKey(dtype, kind, row.logNi[i], row.BS[i], row.n[i], int(ft), int(row.split[i]) if row.split else 0,
-                      int(row.pf[i]) if row.pf else 0)
+                      int(row.pf[i]) if row.pf else 0,
+                      # fault-tolerant plans keep the LDS path: the checksum model fixes which
+                      # outputs a thread owns
+                      (int(row.xl[i]) if row.xl else 0) if not ft else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 
 

@@ -45,6 +45,10 @@ extern long long tfft_sim_errors;
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
+// cross-lane fetch in the lock-step flavour: the partner's registers as snapshotted
+// before the stage
+#define XLANE(i, MASK, dst) { dst = ts[tx ^ (MASK)].sh[i]; }
+#define SNAP() { for (unsigned z_ = 0; z_ < sizeof(ts[tx].sh) / sizeof(ts[tx].sh[0]); ++z_) ts[tx].sh[z_] = r[z_]; }
 #endif
 
 TFFT_DEV float2 cadd(float2 a, float2 b) { float2 c; c.x = a.x + b.x; c.y = a.y + b.y; return c; }
@@ -66,6 +70,23 @@ TFFT_DEV double2 cneg(double2 a) { double2 c; c.x = -a.x; c.y = -a.y; return c; 
 TFFT_DEV double2 czero(double2) { double2 c; c.x = 0.0; c.y = 0.0; return c; }
 
 #ifndef TFFT_SIM
+// Cross-lane fetch of the value held by lane (lane ^ MASK): DPP quad permutes for
+// MASK 1 and 2, the ds_swizzle crossbar (bit mode, no LDS memory touched) for 4.
+template <int MASK> TFFT_DEV int xl_i32(int v) {
+    static_assert(MASK == 1 || MASK == 2 || MASK == 4, "cross-lane distance");
+    if (MASK == 1) return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);        // quad_perm [1,0,3,2]
+    if (MASK == 2) return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);        // quad_perm [2,3,0,1]
+    return __builtin_amdgcn_ds_swizzle(v, 0x101F);                                   // and 0x1f, or 0, xor 4
+}
+template <int MASK> TFFT_DEV float xl_r(float v) { return __int_as_float(xl_i32<MASK>(__float_as_int(v))); }
+template <int MASK> TFFT_DEV double xl_r(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = xl_i32<MASK>((int)(b & 0xffffffffll)), hi = xl_i32<MASK>((int)(b >> 32));
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+#define XLANE(i, MASK, dst) { dst.x = xl_r<MASK>(r[i].x); dst.y = xl_r<MASK>(r[i].y); }
+#define SNAP()
+
 // Sum over the 64 lanes of a wavefront; every lane receives the total.
 // Steps 1 and 2 are DPP quad permutes, 4/8/16 go through the ds_swizzle
 // crossbar (no LDS memory is touched), 32 uses a permute across the two halves.
