@@ -22,6 +22,9 @@
 #define TWLD(p, i) ((p)[(i)])
 #define LLD(i) (lds[(i)])
 #define LST(i, v) (lds[(i)] = (v))
+// makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
+// tile-independent table reads inside the tile loop instead of hoisted into registers
+#define OPAQUE(v) asm volatile("" : "+v"(v))
 #else
 #include <cmath>
 #include <cstdio>
@@ -43,6 +46,7 @@ extern long long tfft_sim_errors;
 #define GLDU(p, ub, off) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)])
 #define GSTU(p, ub, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)] = (v))
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
+#define OPAQUE(v)
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
 // cross-lane fetch in the lock-step flavour: the partner's registers as snapshotted
