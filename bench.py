@@ -70,7 +70,7 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
         "gbs": plan.gbs(bs, wall_ms), "gflops": plan.gflops(bs, wall_ms),
         "alg_bytes": plan.algorithmic_bytes(bs),
     }
-    if if_ft:
+    if if_ft or if_err:
         res["ft"] = {k: v for k, v in plan.ft_counters().items() if k != "flagged"}
     plan.close()
     return res, x, out
@@ -195,13 +195,13 @@ def main():
         "gflops": r["gflops"],
         "config": {"workload": f"forward C2C FFT {tname} N=2^{logN} batch=2^{int(math.log2(bs))} "
                                f"({launches}-launch plan {r['plan']['logNi']}, BS {r['plan']['BS']}, n {r['plan']['n']})"
-                               + (", fault tolerant" if a.if_ft else ""),
+                               + (", fault tolerant" if (a.if_ft or a.if_err) else ""),
                    "logN": logN, "bs": bs, "if_ft": a.if_ft, "if_err": a.if_err, "thread_bs": a.thread_bs},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel_ms": kernel_ms, "alg_bytes_per_launch": r["alg_bytes"]},
     }
-    if a.if_ft:
+    if a.if_ft or a.if_err:
         line["ft"] = r.get("ft")
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(logN, dt, a.cpu_seconds)

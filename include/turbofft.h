@@ -109,7 +109,8 @@ int turbofft_set_ft_params(turbofft_plan_t* plan, double err_smoothing, double e
  *   mode 0  none
  *   mode 1  reference cadence: in every `every`-th block, the tile with
  *           cnt == block % thread_bs + 1 gets `mag` added to re of element
- *           (s, m) after the input checksum (s = m = 0 in the reference)
+ *           (s, m) after the input checksum (s = m = 0 in the reference);
+ *           m is limited to the first Ni/n elements of the sub-FFT
  *   mode 2  tiles with tile % every == tile_phase                              */
 int turbofft_set_injection(turbofft_plan_t* plan, int mode, int launch, int every,
                            long long tile_phase, int s, int m, double mag);

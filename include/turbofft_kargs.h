@@ -33,7 +33,7 @@ typedef struct tfft_ft_args {
     int inj_every;
     long long inj_tile;
     int inj_s;                    /* sub-FFT inside the tile                               */
-    int inj_m;                    /* element of that sub-FFT                               */
+    int inj_m;                    /* element of that sub-FFT, 0 <= inj_m < Ni/n            */
     double inj_mag;               /* added to the real part after the input checksum       */
     double err_smoothing;         /* |delta| / (err_smoothing + |mag|) > err_threshold     */
     double err_threshold;

@@ -57,10 +57,13 @@ def build_sim(spec: KernelSpec):
     os.makedirs(_CACHE, exist_ok=True)
     so = os.path.join(_CACHE, f"{spec.name}_{h}.so")
     if not os.path.exists(so):
-        cpp = so[:-3] + ".cpp"
-        with open(cpp, "w") as f:
+        # build under a private name and rename: parallel test workers may want the same library
+        tmp = f"{so[:-3]}.{os.getpid()}"
+        with open(tmp + ".cpp", "w") as f:
             f.write(src)
-        subprocess.check_call(["g++", "-O1", "-shared", "-fPIC", "-o", so, cpp])
+        subprocess.check_call(["g++", "-O1", "-shared", "-fPIC", "-o", tmp + ".so", tmp + ".cpp"])
+        os.replace(tmp + ".so", so)
+        os.remove(tmp + ".cpp")
     return C.CDLL(so)
 
 

@@ -89,7 +89,7 @@ def test_host_chosen_injection_single_tile():
     # mode 2: one tile in the whole run, arbitrary element
     ntiles, tbs, gap = 20, 5, 2
     sp, x, y, c, fl = run_ft("float2", 8, 4, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000,
-                             inj_tile=13, inj_s=2, inj_m=77, mag=100.0)
+                             inj_tile=13, inj_s=2, inj_m=11, mag=100.0)
     assert c[1] == 1 and c[2] == 1 and fl == [(0, 13)]
     assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("float2", 8)
 

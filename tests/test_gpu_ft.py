@@ -144,7 +144,7 @@ def test_threshold_rule():
 def test_injection_in_an_earlier_launch_is_caught_there():
     plan = turbofft_amd.TurboFFT(15, "double2", if_ft=1, thread_bs=2)
     plan.set_ft_params(1000.0, 1e-3, correct=True)
-    plan.set_injection(2, launch=0, every=1 << 30, tile_phase=9, s=3, m=17, mag=100.0)
+    plan.set_injection(2, launch=0, every=1 << 30, tile_phase=9, s=3, m=1, mag=1000.0)
     x = make(4, 1 << 15, "double2", 5)
     y, c = run(plan, x)
     assert c["flagged"] == [(0, 9)] and c["corrected"] == 1
@@ -228,3 +228,12 @@ def test_config5_fp64_2p20_batch256():
             for b in ref_idx:
                 assert O.rel_l2(y[b].cpu().numpy(), O.fft_ref(xsel[b])) <= O.tolerance("double2", logN)
     assert len(model) == len(inj_tiles)          # the sized error is caught in every group
+
+
+def test_injection_element_is_validated():
+    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1)       # Ni = 1024, n = 8: m < 128
+    plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=127)
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=128)
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        plan.set_injection(2, every=1 << 30, tile_phase=0, s=1, m=0)

@@ -25,6 +25,8 @@
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
 // tile-independent table reads inside the tile loop instead of hoisted into registers
 #define OPAQUE(v) asm volatile("" : "+v"(v))
+// instruction-scheduling fence: nothing may be moved across it
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 #else
 #include <cmath>
 #include <cstdio>
@@ -47,6 +49,7 @@ extern long long tfft_sim_errors;
 #define GSTU(p, ub, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)] = (v))
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
 #define OPAQUE(v)
+#define SCHED_FENCE()
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
 // cross-lane fetch in the lock-step flavour: the partner's registers as snapshotted

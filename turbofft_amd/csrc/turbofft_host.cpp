@@ -443,8 +443,9 @@ int turbofft_set_injection(turbofft_plan_t* p, int mode, int launch, int every, 
     if (mode < 0 || mode > 2 || every < 1) return fail(TURBOFFT_EINVAL, "bad injection mode/every");
     int li = launch < 0 ? p->launches - 1 : launch;
     if (li >= p->launches) return fail(TURBOFFT_EINVAL, "bad injection launch");
-    if (s < 0 || s >= p->row.BS(li) || m < 0 || m >= (1 << p->row.logNi(li)))
-        return fail(TURBOFFT_EINVAL, "injection element (s=%d, m=%d) outside the tile", s, m);
+    if (s < 0 || s >= p->row.BS(li) || m < 0 || m >= (1 << p->row.logNi(li)) / p->row.n(li))
+        return fail(TURBOFFT_EINVAL, "injection element (s=%d, m=%d): need 0 <= s < BS=%d and 0 <= m < Ni/n=%d", s, m,
+                    p->row.BS(li), (1 << p->row.logNi(li)) / p->row.n(li));
     if (mode == 2 && (tile_phase < 0 || tile_phase >= every)) return fail(TURBOFFT_EINVAL, "tile_phase must be in [0, every)");
     p->inj_mode = mode; p->inj_launch = launch; p->inj_every = every; p->inj_tile = tile_phase;
     p->inj_s = s; p->inj_m = m; p->inj_mag = mag;
