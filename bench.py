@@ -27,6 +27,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
+# what the same counter reads for a plain 2 GiB copy (2.000 and 1.000 KiB per count); the runs are
+# listed in profiles/.  Keyed by (datatype, logN, bs, fault tolerant); other workloads report null.
+MEASURED_TRAFFIC = {
+    (0, 13, 1 << 15, 0): 4362440823,     # tfft_f32_row1_N13_b1_n32_s_w3: 1.0157 x algorithmic (one spilled register)
+    (0, 16, 1 << 12, 0): 4295128267,     # tfft_f32_col_N7_b32_n32 / tfft_f32_rowT_N9_b16_n32, either launch
+}
 
 
 def make_input(torch, bs, N, datatype, seed=0):
@@ -198,7 +205,8 @@ def main():
                                + (", fault tolerant" if (a.if_ft or a.if_err) else ""),
                    "logN": logN, "bs": bs, "if_ft": a.if_ft, "if_err": a.if_err, "thread_bs": a.thread_bs},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC.get((dt, logN, bs, int(bool(a.if_ft or a.if_err)))),
                      "kernel_ms": kernel_ms, "alg_bytes_per_launch": r["alg_bytes"]},
     }
     if a.if_ft or a.if_err:

@@ -55,6 +55,23 @@ def test_builtin_rows_match_csv_and_are_consistent(dtype):
         turbofft_amd.builtin_plan_row(dtype, 40)
 
 
+def test_optional_plan_columns():
+    """Columns beyond the reference's 11: per-launch split / prefetch / cross-lane flags,
+    tiles per block, per-launch wavefronts per SIMD.  Shorter rows mean zeros."""
+    from turbofft_amd.codegen.fft_codegen import generate_source
+    r = P.PlanRow.from_list([19, 2, 9, 10, 0, 32, 16, 0, 32, 32, 0, 1, 1, 0, 0, 0, 0, 0, 0, 0, 8, 4, 3])
+    assert (r.split, r.pf, r.xl, r.tiles, r.wv) == ((1, 1), (0, 0), (0, 0), 8, (4, 3))
+    plain = P.kernels_for_row(r, "float2", 0)
+    assert [k.name for k in plain] == ["tfft_f32_col_N9_b32_n32_s_w4", "tfft_f32_rowT_N10_b16_n32_s_w3"]
+    # the register budget hint and the cross-lane pass belong to the plain kernels only
+    assert [k.name for k in P.kernels_for_row(r, "float2", 1)] == ["tfft_f32_col_N9_b32_n32_s_ft", "tfft_f32_rowT_N10_b16_n32_s_ft"]
+    src = generate_source([KernelSpec(plain[0])], False)
+    assert "amdgpu_waves_per_eu(4, 4)" in src
+    short = P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0])
+    assert (short.split, short.tiles, short.wv) == ((0,), 0, (0,))
+    assert "amdgpu_waves_per_eu" not in generate_source([KernelSpec(P.kernels_for_row(short, "float2", 0)[0])], False)
+
+
 @pytest.mark.parametrize("dtype", ["float2", "double2"])
 def test_twiddle_table_matches_oracle(dtype):
     a = turbofft_amd.twiddle_table(1 << 12, dtype)

@@ -693,7 +693,8 @@ class KernelEmitter:
             c(f"std::vector<{LT}> ldsv({sp.lds_elems}); {LT}* lds = ldsv.data();")
             c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
         else:
-            c(f'extern "C" __global__ __launch_bounds__({sp.threads})')
+            wv = int(sp.key.wv)
+            c(f'extern "C" __global__ __launch_bounds__({sp.threads})' + (f" __attribute__((amdgpu_waves_per_eu({wv}, {wv})))" if wv else ""))
             c(f"void {sp.name}(const {T2}* __restrict__ in, {T2}* __restrict__ out, const {T2}* __restrict__ tw, const tfft_kargs a)")
             c("{")
             c.ind += 1
@@ -880,7 +881,7 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     kinds = {"row1": 0, "col": 1, "rowT": 2}
     for sp in specs:
         k = sp.key
-        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {sp.threads}, {sp.lds_bytes}}},')
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {int(k.wv)}, {sp.threads}, {sp.lds_bytes}}},')
     c("};")
     c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")

@@ -6,7 +6,11 @@ A plan CSV keeps the reference's 11-column row
 row index == logN.  Three optional trailing columns `x1, x2, x3` select, per
 launch, the split exchange (re and im go through a half-size LDS buffer in two
 rounds), three more `p1, p2, p3` the next-tile prefetch and three more
-`c1, c2, c3` the cross-lane last pass; a row without them means all zeros.  Launch i transforms a digit of size 2^logNi with BSi
+`c1, c2, c3` the cross-lane last pass; a row without them means all zeros.  A
+21st column is the number of tiles a block of a plain (not fault-tolerant) plan
+walks when the caller leaves thread_bs at 1 (0 or absent: one); columns 22-24
+`w1, w2, w3` ask the compiler to fit that many wavefronts per SIMD (0: its own
+choice) for the plain kernel of the launch.  Launch i transforms a digit of size 2^logNi with BSi
 sub-FFTs per tile and ni elements per thread; launch 0 owns the most-strided
 digit and the last launch the contiguous one.
 """
@@ -26,6 +30,8 @@ class PlanRow:
     split: Tuple[int, ...] = ()      # optional columns 12-14: 1 = exchange re and im separately
     pf: Tuple[int, ...] = ()         # optional columns 15-17: 1 = prefetch the next tile
     xl: Tuple[int, ...] = ()         # optional columns 18-20: 1 = last small-radix pass across lanes
+    tiles: int = 0                   # optional column 21: tiles per block of the plain plan (0 = 1)
+    wv: Tuple[int, ...] = ()         # optional columns 22-24: wavefronts per SIMD to compile for (0 = free)
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -39,7 +45,8 @@ class PlanRow:
         ext2 = (row[14:17] + [0, 0, 0])[:3]
         ext3 = (row[17:20] + [0, 0, 0])[:3]
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
-                    tuple(ext2[:L]), tuple(ext3[:L]))
+                    tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
+                    tuple((row[21:24] + [0, 0, 0])[:L]))
         if L and sum(p.logNi) != p.logN:
             raise ValueError(f"logN1+logN2+logN3 != logN in row {row}")
         return p
@@ -60,12 +67,13 @@ class KernelKey:
     split: int = 0   # 1: every LDS exchange moves re and im in two rounds through a half-size buffer
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
+    wv: int = 0      # > 0: compiled to fit this many wavefronts per SIMD (register budget 512 / wv)
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
-                + ("_ft" if self.ft else ""))
+                + (f"_w{self.wv}" if self.wv else "") + ("_ft" if self.ft else ""))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:
@@ -75,7 +83,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:20] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:24] if t.strip()]))
     return rows
 
 
@@ -88,7 +96,9 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
                       int(row.pf[i]) if row.pf else 0,
                       # fault-tolerant plans keep the LDS path: the checksum model fixes which
                       # outputs a thread owns
-                      (int(row.xl[i]) if row.xl else 0) if not ft else 0)
+                      (int(row.xl[i]) if row.xl else 0) if not ft else 0,
+                      # the register budget hint was tuned on the plain kernel only
+                      (int(row.wv[i]) if row.wv else 0) if not ft else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 
 

@@ -47,8 +47,11 @@ constexpr double kPi = 3.14159265358979323846;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[20];           // 11 reference columns + optional per-launch flags: split exchange,
-                         // prefetch, cross-lane last pass
+    int v[24];           // 11 reference columns + optional per-launch flags: split exchange,
+                         // prefetch, cross-lane last pass; then the tiles-per-block hint and
+                         // the per-launch wavefronts-per-SIMD the kernel was compiled for
+    int tiles() const { return v[20]; }
+    int wv(int i) const { return v[21 + i]; }
     int split(int i) const { return v[11 + i]; }
     int pf(int i) const { return v[14 + i]; }
     int xl(int i) const { return v[17 + i]; }
@@ -70,7 +73,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 20 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 24 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -82,12 +85,12 @@ int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
     return i == launches - 1 ? 2 : 1;
 }
 
-const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl) {
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv) {
     int cnt = 0;
     const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
-            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl)
+            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv)
             return &t[i];
     return nullptr;
 }
@@ -271,6 +274,11 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     const Row& r = p->row;
     if (r.logN() != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row %d describes logN=%d", p->logN, r.logN());
     p->launches = r.launches();
+    // Without checksums the number of tiles a block walks is a pure tuning knob: a caller that
+    // leaves thread_bs at its default gets the value tuned for this size (large tiles amortise
+    // the block launch over several of them).  With fault tolerance thread_bs is the checksum
+    // group size and stays what the caller asked for.
+    if (!p->if_ft && p->thread_bs == 1 && r.tiles() > 1) p->thread_bs = r.tiles();
     int sum = 0;
     for (int i = 0; i < p->launches; ++i) sum += r.logNi(i);
     if (sum != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row for logN=%d: digit sizes sum to %d", p->logN, sum);
@@ -285,7 +293,8 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     for (int i = 0; i < p->launches; ++i) {
         int kind = kind_of_launch(p->launches, i);
         const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
-                                                 (r.xl(i) && !p->if_ft) ? 1 : 0);   // FT plans keep the LDS path
+                                                 (r.xl(i) && !p->if_ft) ? 1 : 0,    // FT plans keep the LDS path
+                                                 p->if_ft ? 0 : r.wv(i));
         if (!k)
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
