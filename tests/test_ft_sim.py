@@ -118,3 +118,19 @@ def test_ft_with_prefetch_recomputes_the_located_tile():
     sp, x, y, c, fl = run_ft("double2", 10, 1, 8, 20, 5, 2, inj_mode=2, correct=1, inj_every=1000, inj_tile=13, pf=1)
     assert c[1] == 1 and c[2] == 1 and fl == [(0, 13)]
     assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 10)
+
+
+def test_table_fetched_ahead_of_the_tile_in_full_lds_kernels():
+    """A block that fills the CU's LDS fetches its checksum-table entries before the tile
+    loads (another instruction order, same arithmetic): decisions and correction as usual."""
+    from turbofft_amd.codegen.fft_codegen import KernelEmitter
+    sp = KernelSpec(KernelKey("double2", "row1", 10, 8, 16, 1))
+    assert KernelEmitter(sp).ft_table_early() and sp.lds_bytes > 80 * 1024
+    assert not KernelEmitter(KernelSpec(KernelKey("double2", "row1", 8, 4, 16, 1))).ft_table_early()
+    ntiles, tbs, gap = 6, 3, 2
+    sp, x, y, c, fl = run_ft("double2", 10, 8, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000,
+                             inj_tile=4, inj_s=5, inj_m=17, mag=1.0e4)
+    assert c[1] == 1 and c[2] == 1 and fl == [(0, 4)]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 10)
+    sp, x, y, c, fl = run_ft("double2", 10, 8, 16, ntiles, tbs, gap, inj_mode=0, correct=1)
+    assert c[1] == 0 and not fl

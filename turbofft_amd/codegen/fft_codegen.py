@@ -470,6 +470,30 @@ class KernelEmitter:
         c("}")
 
     # ---------- fault tolerance ----------
+    def ft_table_early(self) -> bool:
+        """Whether a thread fetches all its checksum-table entries before its tile data
+        (needs 2n more live registers while the tile loads are in flight)."""
+        # pays when one block fills the CU's LDS: nothing else is resident to cover the wait
+        # for the table after the data, and there are registers to spare
+        return self.s.threads < 1024 and self.s.lds_bytes > 80 * 1024
+
+    def emit_ft_table_load(self, c: Code):
+        """Issue the loads of this thread's n table entries ahead of the tile loads: the
+        table is L2-resident, so its latency hides behind the HBM latency of the data
+        and the checksum accumulates as the elements arrive."""
+        sp = self.s
+        c("unsigned xc = x;")
+        if sp.n * (2 if self.R == "float" else 4) > 32:
+            # the table entries of a thread are the same for every tile; with many elements per
+            # thread keeping them all in registers across the loop costs more than re-reading
+            c("OPAQUE(xc);")
+        if not self.ft_table_early():
+            return
+        c(f"{self.T2} cv[{sp.n}];")
+        for e in range(sp.n):
+            c(f"cv[{e}] = TWLD(ck, xc + {sp.Tr * e}u);")
+        c("SCHED_FENCE();")
+
     def emit_ft_input(self, c: Code):
         """in1 += re+im of x*c[m]; in2 += cnt * (...)   (fft_codegen.py:354-367),
         then the optional compute-side error injection (:412-415).
@@ -479,23 +503,23 @@ class KernelEmitter:
         c("if (!is_redo) {")
         c.ind += 1
         c(f"{self.R} acc = 0;")
-        c("unsigned xc = x;")
-        if sp.n * (2 if self.R == "float" else 4) > 32:
-            # the table entries of a thread are the same for every tile; with many elements per
-            # thread keeping them all in registers across the loop costs more than re-reading
-            c("OPAQUE(xc);")
-        # The table is fetched in batches: every load of a batch is issued back to back and
-        # waited for once.  Left to itself the compiler alternates load / wait / use per
-        # element, a chain of n L2 round trips per tile (+80 % run time at 8192 points).
-        B = 8 if sp.threads >= 1024 else min(sp.n, 16 if self.R == "double" else 32)
-        c(f"{self.T2} cv[{B}];")
-        for b0 in range(0, sp.n, B):
-            for e in range(b0, min(sp.n, b0 + B)):
-                c(f"cv[{e - b0}] = TWLD(ck, xc + {sp.Tr * e}u);")
-            c("SCHED_FENCE();")
-            for e in range(b0, min(sp.n, b0 + B)):
-                c(f"acc += r[{e}].x * cv[{e - b0}].x + r[{e}].y * cv[{e - b0}].y;")
-            c("SCHED_FENCE();")
+        if self.ft_table_early():
+            for e in range(sp.n):
+                c(f"acc += r[{e}].x * cv[{e}].x + r[{e}].y * cv[{e}].y;")
+        else:
+            # The table is fetched after the data in batches (8 entries where 1024-thread blocks
+            # leave 128 registers per lane), every load of a batch issued back to back and
+            # waited for once.  Left to itself the compiler alternates load / wait / use per element, a
+            # chain of n L2 round trips per tile.
+            B = 8 if sp.threads >= 1024 else min(sp.n, 16 if self.R == "double" else 32)
+            c(f"{self.T2} cv[{B}];")
+            for b0 in range(0, sp.n, B):
+                for e in range(b0, min(sp.n, b0 + B)):
+                    c(f"cv[{e - b0}] = TWLD(ck, xc + {sp.Tr * e}u);")
+                c("SCHED_FENCE();")
+                for e in range(b0, min(sp.n, b0 + B)):
+                    c(f"acc += r[{e}].x * cv[{e - b0}].x + r[{e}].y * cv[{e - b0}].y;")
+                c("SCHED_FENCE();")
         c("fin1 += acc; fin2 += cntf * acc;")
         # the injected element is one of the first Ni/n of its sub-FFT (register 0 of thread
         # x = m; the reference injects at m = 0)
@@ -610,6 +634,7 @@ class KernelEmitter:
                     for e in range(sp.n):
                         c(f"r[{e}] = rn[{e}];")
                     if sp.ft:
+                        self.emit_ft_table_load(c)
                         self.emit_ft_input(c)
                     c("if (has_next) {")
                     c.ind += 1
@@ -618,6 +643,8 @@ class KernelEmitter:
                     c.ind -= 1
                     c("}")
                 else:
+                    if sp.ft:
+                        self.emit_ft_table_load(c)
                     self.emit_load(c)
                     if sp.ft:
                         self.emit_ft_input(c)
