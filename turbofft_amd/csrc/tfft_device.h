@@ -13,13 +13,45 @@
 #ifndef TFFT_SIM
 #include <hip/hip_runtime.h>
 #define TFFT_DEV __device__ __forceinline__
-#define GLD(p, i) ((p)[(i)])
-#define GST(p, i, v) ((p)[(i)] = (v))
-// wave-uniform 64-bit base + 32-bit per-lane offset: lets the compiler keep the base in
-// SGPRs (saddr addressing) so an access costs no vector address arithmetic
-#define GLDU(p, ub, off) (((p) + (ub))[(off)])
-#define GSTU(p, ub, off, v) (((p) + (ub))[(off)] = (v))
-#define TWLD(p, i) ((p)[(i)])
+// Global memory goes through buffer instructions: the resource holds a wave-uniform base
+// (tensor pointer + tile base, SGPRs), a second uniform offset rides in an SGPR and the lane
+// part is ONE 32-bit VGPR shared by every access of a tile -- no per-access vector address
+// arithmetic and no 64-bit address registers.  (p, ub): uniform element base; uo: uniform
+// element offset; off / i: per-lane element offset.  All offsets within a tile or table are
+// below 2^32 bytes.
+typedef unsigned tfft_u2 __attribute__((ext_vector_type(2)));
+typedef unsigned tfft_u4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tfft_rsrc(const void* p) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, -1, 0x00020000);
+}
+__device__ __forceinline__ float2 tfft_bld(const float2* p, unsigned voff, unsigned soff) {
+    const tfft_u2 t = __builtin_amdgcn_raw_buffer_load_b64(tfft_rsrc(p), voff, soff, 0);
+    float2 r; r.x = __uint_as_float(t.x); r.y = __uint_as_float(t.y); return r;
+}
+__device__ __forceinline__ double2 tfft_bld(const double2* p, unsigned voff, unsigned soff) {
+    const tfft_u4 t = __builtin_amdgcn_raw_buffer_load_b128(tfft_rsrc(p), voff, soff, 0);
+    double2 r; r.x = __hiloint2double((int)t.y, (int)t.x); r.y = __hiloint2double((int)t.w, (int)t.z); return r;
+}
+__device__ __forceinline__ void tfft_bst(float2* p, unsigned voff, unsigned soff, float2 v) {
+    tfft_u2 t; t.x = __float_as_uint(v.x); t.y = __float_as_uint(v.y);
+    __builtin_amdgcn_raw_buffer_store_b64(t, tfft_rsrc(p), voff, soff, 0);
+}
+__device__ __forceinline__ void tfft_bst(double2* p, unsigned voff, unsigned soff, double2 v) {
+    tfft_u4 t;
+    t.x = (unsigned)__double2loint(v.x); t.y = (unsigned)__double2hiint(v.x);
+    t.z = (unsigned)__double2loint(v.y); t.w = (unsigned)__double2hiint(v.y);
+    __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, 0);
+}
+#define TFFT_ESZ(p) ((unsigned)sizeof(*(p)))
+#define GLDU(p, ub, uo, off) tfft_bld((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
+#define GSTU(p, ub, uo, off, v) tfft_bst((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
+// plain global-pointer forms of the same accesses
+#define GLDG(p, ub, uo, off) (((p) + ((ub) + (uo)))[(off)])
+#define GSTG(p, ub, uo, off, v) (((p) + ((ub) + (uo)))[(off)] = (v))
+#define TWLG(p, i) ((p)[(i)])
+#define TWLGU(p, c, i) ((p)[(c) + (i)])
+#define TWLD(p, i) tfft_bld((p), (unsigned)(i) * TFFT_ESZ(p), 0u)
+#define TWLDU(p, c, i) tfft_bld((p), (unsigned)(i) * TFFT_ESZ(p), (unsigned)(c) * TFFT_ESZ(p))
 #define LLD(i) (lds[(i)])
 #define LST(i, v) (lds[(i)] = (v))
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
@@ -43,11 +75,14 @@ extern long long tfft_sim_errors;
          ? (tfft_sim_errors++ == 0 ? fprintf(stderr, "tfft sim: %s index %lld out of [0,%lld) at %s:%d\n", \
                                              what, (long long)(i), (long long)(n), __FILE__, __LINE__) : 0, 0LL) \
          : (long long)(i))
-#define GLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
-#define GST(p, i, v) ((p)[TFFT_CHK((i), p##_limit, #p)] = (v))
-#define GLDU(p, ub, off) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)])
-#define GSTU(p, ub, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(off), p##_limit, #p)] = (v))
+#define GLDU(p, ub, uo, off) ((p)[TFFT_CHK((long long)(ub) + (long long)(uo) + (long long)(off), p##_limit, #p)])
+#define GSTU(p, ub, uo, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(uo) + (long long)(off), p##_limit, #p)] = (v))
+#define GLDG(p, ub, uo, off) GLDU(p, ub, uo, off)
+#define GSTG(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
+#define TWLG(p, i) TWLD(p, i)
+#define TWLGU(p, c, i) TWLDU(p, c, i)
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
+#define TWLDU(p, c, i) ((p)[TFFT_CHK((long long)(c) + (long long)(i), p##_limit, #p)])
 #define OPAQUE(v)
 #define SCHED_FENCE()
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
