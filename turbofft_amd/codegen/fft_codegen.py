@@ -207,10 +207,20 @@ class KernelEmitter:
         xn = "x"
         if sp.xl and q == sp.npass_lds - 1:
             xn = "xraw"
+        t = "tx"
+        if sp.threads >= 1024:
+            # Everything derived from the thread index (LDS addresses, table indices, lane
+            # offsets) is the same for every tile, and LLVM hoists it all out of the tile loop:
+            # dozens of registers live across the whole kernel, 20-60 of them spilled under the
+            # 128-register cap of a 1024-thread block.  An opaque copy per phase makes each phase
+            # recompute its few shifts and masks instead (kernels with room for the hoisted
+            # values measured 2-6 % slower that way and keep the plain index).
+            c("unsigned txq = tx; OPAQUE(txq);")
+            t = "txq"
         if sp.maps[q] == "major":
-            c(f"const unsigned s = tx >> {ilog2(sp.Tr)}, {xn} = tx & {sp.Tr - 1}u;")
+            c(f"const unsigned s = {t} >> {ilog2(sp.Tr)}, {xn} = {t} & {sp.Tr - 1}u;")
         else:
-            c(f"const unsigned s = tx & {sp.BS - 1}u, {xn} = tx >> {ilog2(sp.BS)};")
+            c(f"const unsigned s = {t} & {sp.BS - 1}u, {xn} = {t} >> {ilog2(sp.BS)};")
         if xn == "xraw":
             # the RL partners of the cross-lane pass are adjacent lanes: sub-index j = xraw % RL,
             # completed digits low = xraw / RL; x is the row position low + P*j the pass works on
