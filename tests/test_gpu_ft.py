@@ -202,10 +202,20 @@ def test_config5_fp64_2p20_batch256():
     need = sorted({t // tpt for gr in hit_groups for t in gr})
     xsel = {b: x[b].cpu().numpy() for b in need}
     ref_idx = need[:3]
+    # An error e on input element m moves delta by e * (re c[m] + im c[m]) but also every output
+    # of the sub-FFT by |e|, i.e. mag by about |e| * Ni / sqrt(n): for long sub-FFTs the ratio
+    # saturates below the threshold and the reference rule cannot fire at any magnitude.  The
+    # model says which regime this plan's last launch is in; the GPU must agree either way.
+    huge = [O.Injection(t, 1, 5, 1e15) for t in inj_tiles]
+    detectable = all(d.detected for d in _model_groups_last_launch(xsel, row, "double2", hit_groups, tpt, huge, tbs))
+    print("config5 plan", plan.logNi, plan.BS, plan.n, "single-element errors detectable in the last launch:", detectable, flush=True)
     for mag in (100.0, None):
         if mag is None:
             clean = _model_groups_last_launch(xsel, row, "double2", hit_groups, tpt, [], tbs)
-            mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean)) / 1.0))
+            cm = O.dft_checksum_vector(1 << plan.logNi[last], "double2")[5]
+            weight = abs(cm.real + cm.imag)
+            assert weight > 1e-6
+            mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean)) / min(weight, 1.0)))
         injs = [O.Injection(t, 1, 5, mag) for t in inj_tiles]
         dec = _model_groups_last_launch(xsel, row, "double2", hit_groups, tpt, injs, tbs)
         for d in dec:
@@ -227,7 +237,8 @@ def test_config5_fp64_2p20_batch256():
         if len(model) == len(inj_tiles):         # everything corrected: transforms must be clean
             for b in ref_idx:
                 assert O.rel_l2(y[b].cpu().numpy(), O.fft_ref(xsel[b])) <= O.tolerance("double2", logN)
-    assert len(model) == len(inj_tiles)          # the sized error is caught in every group
+    # the sized error is caught in every group, unless the rule cannot see it at all
+    assert len(model) == (len(inj_tiles) if detectable else 0)
 
 
 def test_injection_element_is_validated():

@@ -273,3 +273,24 @@ def test_metrics_formulas():
     # 2^28 points fp32 in 3.120 ms -> the reference's published 5592 GFLOPS, 1376.5 GB/s
     assert math.isclose(O.gflops(1 << 13, 1 << 15, 3.120), 5592.0, rel_tol=1e-3)
     assert math.isclose(O.algorithmic_gbs(1 << 13, 1 << 15, 3.120, "float2"), 1376.5, rel_tol=1e-3)
+
+
+def test_rule_saturates_for_long_subffts():
+    """An input error e moves delta by e*(re c[m] + im c[m]) and mag by about
+    |e|*Ni/sqrt(n) (every output of the sub-FFT is off by |e|): the ratio the reference rule
+    tests tends to a constant as e grows -- above the 1e-3 threshold for a 256-point
+    sub-FFT, below it for a 2048-point one, which therefore cannot flag such an error."""
+    rng = np.random.default_rng(5)
+    seen = {}
+    for Ni, n in ((256, 16), (2048, 16)):
+        x = (rng.uniform(-1, 1, (4, 1, Ni)) + 1j * rng.uniform(-1, 1, (4, 1, Ni)))
+        cv = O.dft_checksum_vector(Ni, "double2")
+        ratios = []
+        for mag in (1e9, 1e12):
+            y = O.fft_ref(x)
+            y[2, 0, :] += mag * np.exp(-2j * np.pi * 5 * np.arange(Ni) / Ni)      # error on x[5] of tile 2
+            d = O.ft_launch_model(x, y, n, [[0, 1, 2, 3]], "double2", cv)[0]
+            ratios.append(abs(d.delta) / (1000.0 + abs(d.mag)))
+            seen[(Ni, mag)] = d.detected
+        assert abs(ratios[0] / ratios[1] - 1) < 1e-3          # saturated: independent of the magnitude
+    assert seen[(256, 1e12)] and not seen[(2048, 1e12)]
