@@ -64,7 +64,7 @@ def test_reference_cadence_matches_oracle_model(dt, logN, bs, tbs):
     for i, g in enumerate(gaps):
         plan.set_tb_gap(i, g)
     x = make(bs, 1 << logN, dt, logN + 1)
-    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row(dt, logN))
+    row = O.PlanRow.from_list(plan.plan_row())
     if logN <= 10:
         mag = 100.0
     else:
@@ -103,7 +103,7 @@ def test_reference_default_magnitude_is_below_the_rule_at_8192_points():
     plan.set_tb_gap(0, 7)
     x = make(32, 1 << 13, "float2", 14)
     y, c = run(plan, x)
-    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row("float2", 13))
+    row = O.PlanRow.from_list(plan.plan_row())
     groups = O.tile_groups(32, 2, 7)
     injs = O.reference_injections(groups, 2, 100.0)
     dec, _ = O.ft_plan_model(x, row, "float2", 2, [7], injs)
@@ -184,8 +184,8 @@ def test_config5_fp64_2p20_batch256():
     torch = _torch()
     logN, bs, tbs = 20, 256, 8
     N = 1 << logN
-    row = O.PlanRow.from_list(turbofft_amd.builtin_plan_row("double2", logN))
     plan = turbofft_amd.TurboFFT(logN, "double2", if_ft=1, thread_bs=tbs)
+    row = O.PlanRow.from_list(plan.plan_row())
     plan.set_ft_params(1000.0, 1e-3, correct=True)
     last = plan.launches - 1
     gap = 64

@@ -33,7 +33,11 @@ def test_registry_has_every_kernel_of_the_builtin_plans():
     have = set(turbofft_amd.kernel_names())
     for dtype in ("float2", "double2"):
         rows = P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}.csv"))
-        for key in collect_keys(rows, dtype, [0, 1]):
+        ft_rows = list(rows)          # fault-tolerant plans: same rows unless param_<T>_ft.csv replaces one
+        for r in P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}_ft.csv")):
+            assert rows[r.logN].launches > 0
+            ft_rows[r.logN] = r
+        for key in collect_keys(rows, dtype, [0]) + collect_keys(ft_rows, dtype, [1]):
             assert key.name in have
 
 

@@ -153,6 +153,12 @@ class TurboFFT:
     __del__ = close
 
     # ---- geometry ----
+    def plan_row(self) -> List[int]:
+        """The 11 reference columns of the row this plan runs (a fault-tolerant plan may use
+        another built-in row than the plain plan of the same size)."""
+        z = lambda v: list(v) + [0] * (3 - len(v))
+        return [self.logN, self.launches] + z(self.logNi) + z(self.BS) + z(self.n)
+
     def out_elems(self, bs: int) -> int:
         """Elements the output buffer must hold (workspace included)."""
         return self.N * bs * (2 if self.launches > 1 else 1)

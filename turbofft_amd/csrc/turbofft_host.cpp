@@ -20,6 +20,7 @@
 #include "tfft_registry.h"
 
 extern "C" const char* tfft_builtin_param_csv(int datatype);   // generated: the gfx950 CSV text
+extern "C" const char* tfft_builtin_param_ft_csv(int datatype);   // generated: rows replaced in FT plans
 
 namespace {
 
@@ -267,6 +268,15 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     } else {
         std::istringstream in(tfft_builtin_param_csv(p->datatype));
         if (!parse_csv(in, rows)) return fail(TURBOFFT_ENOPLAN, "built-in plan table is malformed");
+        if (p->if_ft) {
+            // the checksum flavour of a kernel needs more registers: where another tile shape
+            // measured faster with checksums, the built-in table carries a replacement row
+            std::istringstream fin(tfft_builtin_param_ft_csv(p->datatype));
+            std::vector<Row> repl;
+            if (!parse_csv(fin, repl)) return fail(TURBOFFT_ENOPLAN, "built-in fault-tolerant plan table is malformed");
+            for (const Row& r : repl)
+                if (r.logN() >= 0 && r.logN() < (int)rows.size()) rows[r.logN()] = r;
+        }
     }
     if (p->logN < 1 || p->logN >= (int)rows.size() || rows[p->logN].launches() < 1 || rows[p->logN].launches() > 3)
         return fail(TURBOFFT_ENOPLAN, "no plan row for logN=%d", p->logN);
