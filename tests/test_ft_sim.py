@@ -120,17 +120,18 @@ def test_ft_with_prefetch_recomputes_the_located_tile():
     assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 10)
 
 
-def test_table_fetched_ahead_of_the_tile_in_full_lds_kernels():
-    """A block that fills the CU's LDS fetches its checksum-table entries before the tile
-    loads (another instruction order, same arithmetic): decisions and correction as usual."""
+def test_table_in_registers_or_read_per_tile():
+    """Blocks of up to 512 threads read their checksum-table entries once and keep them for
+    all their tiles; 1024-thread blocks (128 registers per lane) re-read them per tile in
+    batches.  Same arithmetic either way: decisions and correction as usual."""
     from turbofft_amd.codegen.fft_codegen import KernelEmitter
-    sp = KernelSpec(KernelKey("double2", "row1", 10, 8, 16, 1))
-    assert KernelEmitter(sp).ft_table_early() and sp.lds_bytes > 80 * 1024
-    assert not KernelEmitter(KernelSpec(KernelKey("double2", "row1", 8, 4, 16, 1))).ft_table_early()
-    ntiles, tbs, gap = 6, 3, 2
-    sp, x, y, c, fl = run_ft("double2", 10, 8, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000,
-                             inj_tile=4, inj_s=5, inj_m=17, mag=1.0e4)
-    assert c[1] == 1 and c[2] == 1 and fl == [(0, 4)]
-    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", 10)
-    sp, x, y, c, fl = run_ft("double2", 10, 8, 16, ntiles, tbs, gap, inj_mode=0, correct=1)
-    assert c[1] == 0 and not fl
+    for logNi, BS, n, resident in ((10, 8, 16, True), (10, 8, 8, False)):
+        sp = KernelSpec(KernelKey("double2", "row1", logNi, BS, n, 1))
+        assert KernelEmitter(sp).ft_table_resident() == resident and (sp.threads < 1024) == resident
+        ntiles, tbs, gap = 6, 3, 2
+        sp, x, y, c, fl = run_ft("double2", logNi, BS, n, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000,
+                                 inj_tile=4, inj_s=5, inj_m=17, mag=1.0e4)
+        assert c[1] == 1 and c[2] == 1 and fl == [(0, 4)]
+        assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", logNi)
+        sp, x, y, c, fl = run_ft("double2", logNi, BS, n, ntiles, tbs, gap, inj_mode=0, correct=1)
+        assert c[1] == 0 and not fl

@@ -487,29 +487,33 @@ class KernelEmitter:
         c("}")
 
     # ---------- fault tolerance ----------
-    def ft_table_early(self) -> bool:
-        """Whether a thread fetches all its checksum-table entries before its tile data
-        (needs 2n more live registers while the tile loads are in flight)."""
-        # pays when one block fills the CU's LDS: nothing else is resident to cover the wait
-        # for the table after the data, and there are registers to spare
-        return self.s.threads < 1024 and self.s.lds_bytes > 80 * 1024
+    def ft_table_resident(self) -> bool:
+        """Whether a thread keeps its n checksum-table entries in registers for all the tiles
+        of its block: they are the same for every tile, so the table is read once per block
+        instead of once per tile (-5..6 % run time).  Not under the 128-register cap of a
+        1024-thread block, where the 2n extra registers spill."""
+        return self.s.threads < 1024
+
+    def emit_ft_table_resident_load(self, c: Code, sim: bool):
+        sp = self.s
+        pre = Code()
+        self.map_vars(pre, 0)
+        for e in range(sp.n):
+            pre(f"cvr[{e}] = {self.TWLU}(ck, {sp.Tr * e}u, x);")
+        pre("(void)s;")
+        c("if (count > 0) {")
+        c.ind += 1
+        self.thread_block(c, sim, pre.text())
+        c.ind -= 1
+        c("}")
 
     def emit_ft_table_load(self, c: Code):
-        """Issue the loads of this thread's n table entries ahead of the tile loads: the
-        table is L2-resident, so its latency hides behind the HBM latency of the data
-        and the checksum accumulates as the elements arrive."""
-        sp = self.s
-        c("unsigned xc = x;")
-        if sp.n * (2 if self.R == "float" else 4) > 32:
-            # the table entries of a thread are the same for every tile; with many elements per
-            # thread keeping them all in registers across the loop costs more than re-reading
-            c("OPAQUE(xc);")
-        if not self.ft_table_early():
+        """Lane index of the per-tile table reads (kernels that do not keep the table in
+        registers).  Opaque, so that the reads stay inside the tile loop."""
+        if self.ft_table_resident():
             return
-        c(f"{self.T2} cv[{sp.n}];")
-        for e in range(sp.n):
-            c(f"cv[{e}] = {self.TWLU}(ck, {sp.Tr * e}u, xc);")
-        c("SCHED_FENCE();")
+        c("unsigned xc = x;")
+        c("OPAQUE(xc);")
 
     def emit_ft_input(self, c: Code):
         """in1 += re+im of x*c[m]; in2 += cnt * (...)   (fft_codegen.py:354-367),
@@ -520,15 +524,15 @@ class KernelEmitter:
         c("if (!is_redo) {")
         c.ind += 1
         c(f"{self.R} acc = 0;")
-        if self.ft_table_early():
+        if self.ft_table_resident():
             for e in range(sp.n):
-                c(f"acc += r[{e}].x * cv[{e}].x + r[{e}].y * cv[{e}].y;")
+                c(f"acc += r[{e}].x * cvr[{e}].x + r[{e}].y * cvr[{e}].y;")
         else:
-            # The table is fetched after the data in batches (8 entries where 1024-thread blocks
-            # leave 128 registers per lane), every load of a batch issued back to back and
-            # waited for once.  Left to itself the compiler alternates load / wait / use per element, a
+            # The table is fetched after the data in batches of 8 (a 1024-thread block leaves
+            # 128 registers per lane), every load of a batch issued back to back and waited for
+            # once.  Left to itself the compiler alternates load / wait / use per element, a
             # chain of n L2 round trips per tile.
-            B = 8 if sp.threads >= 1024 else min(sp.n, 16 if self.R == "double" else 32)
+            B = 8
             c(f"{self.T2} cv[{B}];")
             for b0 in range(0, sp.n, B):
                 for e in range(b0, min(sp.n, b0 + B)):
@@ -729,7 +733,7 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx;")
@@ -753,6 +757,8 @@ class KernelEmitter:
                 c(f"{T2} rn[{sp.n}];")
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
+                if self.ft_table_resident():
+                    c(f"{T2} cvr[{sp.n}];")
         # XCD-aware renumbering: hardware deals blocks round-robin to the 8 XCDs, so block
         # b runs on XCD b % 8.  Give every XCD chunks of `xcd_chunk` consecutive tiles (its
         # L2 then streams contiguous memory) while the 8 XCDs stay in one neighbourhood.
@@ -786,6 +792,8 @@ class KernelEmitter:
             c("}")
         if sp.ft:
             c("long long redo_tile = -1; int extra = 0;")
+            if self.ft_table_resident():
+                self.emit_ft_table_resident_load(c, sim)
             c("for (int it = 0; it < count + extra; ++it) {")
             c.ind += 1
             c("const bool is_redo = it >= count;")
@@ -841,8 +849,8 @@ class KernelEmitter:
         if sim:
             c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
             c.ind += 1
-            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
-            c("(void)r; (void)rn; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
+            c("(void)r; (void)rn; (void)cvr; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
         else:
             c("{")
             c.ind += 1
