@@ -208,13 +208,14 @@ class KernelEmitter:
         if sp.xl and q == sp.npass_lds - 1:
             xn = "xraw"
         t = "tx"
-        if sp.threads >= 1024:
+        if sp.threads >= 1024 or sp.n * (2 if self.R == "float" else 4) >= 128:
             # Everything derived from the thread index (LDS addresses, table indices, lane
             # offsets) is the same for every tile, and LLVM hoists it all out of the tile loop:
             # dozens of registers live across the whole kernel, 20-60 of them spilled under the
             # 128-register cap of a 1024-thread block.  An opaque copy per phase makes each phase
             # recompute its few shifts and masks instead (kernels with room for the hoisted
-            # values measured 2-6 % slower that way and keep the plain index).
+            # values measured 2-6 % slower that way and keep the plain index).  Kernels whose
+            # elements alone fill 128 registers per lane get the same treatment.
             c("unsigned txq = tx; OPAQUE(txq);")
             t = "txq"
         if sp.maps[q] == "major":
@@ -491,8 +492,9 @@ class KernelEmitter:
         """Whether a thread keeps its n checksum-table entries in registers for all the tiles
         of its block: they are the same for every tile, so the table is read once per block
         instead of once per tile (-5..6 % run time).  Not under the 128-register cap of a
-        1024-thread block, where the 2n extra registers spill."""
-        return self.s.threads < 1024
+        1024-thread block, where the extra registers spill, nor when the entries alone would
+        take more than 64 registers."""
+        return self.s.threads < 1024 and self.s.n * (2 if self.R == "float" else 4) <= 64
 
     def emit_ft_table_resident_load(self, c: Code, sim: bool):
         sp = self.s
