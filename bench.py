@@ -137,7 +137,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (batches shard trivially across "
-              "GPUs; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "GPUs by splitting the batch, no exchange needed). Run with --gpus 1.", file=sys.stderr)
         return 2
     import torch
     import turbofft_amd
