@@ -242,9 +242,10 @@ def test_config5_fp64_2p20_batch256():
 
 
 def test_injection_element_is_validated():
-    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1)       # Ni = 1024, n = 8: m < 128
-    plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=127)
+    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1)
+    lim = (1 << plan.logNi[-1]) // plan.n[-1]            # the injected element is one of the first Ni/n
+    plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=lim - 1)
     with pytest.raises(turbofft_amd.TurboFFTError):
-        plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=128)
+        plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=lim)
     with pytest.raises(turbofft_amd.TurboFFTError):
-        plan.set_injection(2, every=1 << 30, tile_phase=0, s=1, m=0)
+        plan.set_injection(2, every=1 << 30, tile_phase=0, s=plan.BS[-1], m=0)

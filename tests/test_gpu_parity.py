@@ -41,13 +41,33 @@ def gpu_fft(plan, x):
     return y.cpu().numpy()
 
 
+SHAPES_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "turbofft_amd", "param", "gfx950")
+
+
 def test_config1_fp64_2p10_batch16():
-    # BASELINE config 1: fp64, N=2^10, batch 16, U[-1,1) seed 0, single launch n=8
-    plan = turbofft_amd.TurboFFT(10, "double2")
-    assert plan.launches == 1 and plan.n == [8]
+    # BASELINE config 1: fp64, N=2^10, batch 16, U[-1,1) seed 0, single launch n=8 -- with the
+    # plan shape the configuration names, and with the built-in row for this size
     x = make(16, 1024, "double2", 0)
-    y = gpu_fft(plan, x)
-    assert O.rel_l2(y, O.fft_ref(x)) <= 1e-13 * 10
+    shaped = turbofft_amd.TurboFFT(10, "double2", param_csv=os.path.join(SHAPES_DIR, "reference_shapes_double2.csv"))
+    assert shaped.launches == 1 and shaped.n == [8]
+    for plan in (shaped, turbofft_amd.TurboFFT(10, "double2")):
+        y = gpu_fft(plan, x)
+        assert O.rel_l2(y, O.fft_ref(x)) <= 1e-13 * 10
+
+
+def test_config3_and_config4_plan_shapes():
+    # BASELINE config 3 (fp64 2^15, two launches 7/8 with BS 16/8, standard normal input) and
+    # config 4 (fp32 2^24, three launches 8/8/8 with BS 16): the named plan shapes on a few
+    # transforms; the full 2^28-point sizes of these plans are covered by the sweeps below
+    rng = np.random.default_rng(3)
+    plan = turbofft_amd.TurboFFT(15, "double2", param_csv=os.path.join(SHAPES_DIR, "reference_shapes_double2.csv"))
+    assert (plan.launches, plan.logNi, plan.BS) == (2, [7, 8], [16, 8])
+    x = (rng.standard_normal((5, 1 << 15)) + 1j * rng.standard_normal((5, 1 << 15))).astype(np.complex128)
+    assert O.rel_l2(gpu_fft(plan, x), O.fft_ref(x)) <= O.tolerance("double2", 15)
+    plan = turbofft_amd.TurboFFT(24, "float2", param_csv=os.path.join(SHAPES_DIR, "reference_shapes_float2.csv"))
+    assert (plan.launches, plan.logNi, plan.BS) == (3, [8, 8, 8], [16, 16, 16])
+    x = make(2, 1 << 24, "float2", 4)
+    assert O.rel_l2(gpu_fft(plan, x), O.fft_ref(x)) <= O.tolerance("float2", 24)
 
 
 @pytest.mark.parametrize("dt", ["float2", "double2"])
