@@ -174,6 +174,49 @@ def test_config2_full_size_fp32_2p13():
     assert abs(ey / (N * ex) - 1) < 1e-5
 
 
+def _full_size_check(torch, plan, dt, logN, bs, normal):
+    """Sampled transforms against the oracle plus two size-independent properties of the
+    whole batch: Parseval, and additivity fft(x + x') = fft(x) + fft(x') on a rolled copy."""
+    N = 1 << logN
+    rdt = torch.float32 if dt == "float2" else torch.float64
+    g = torch.Generator(device="cuda").manual_seed(0)
+    if normal:
+        x = torch.randn((bs, N, 2), generator=g, device="cuda", dtype=rdt)
+    else:
+        x = torch.rand((bs, N, 2), generator=g, device="cuda", dtype=rdt) * 2 - 1
+    x = torch.view_as_complex(x)
+    y = plan.fft(x).clone()
+    torch.cuda.synchronize()
+    idx = sorted({0, 1, bs // 3, bs // 2, bs - 1})
+    ref = O.fft_ref(x[idx].cpu().numpy())
+    ys = y[idx].cpu().numpy()
+    for i in range(len(idx)):
+        assert O.rel_l2(ys[i], ref[i]) <= O.tolerance(dt, logN)
+    ex = float((x.real.double() ** 2 + x.imag.double() ** 2).sum())
+    ey = float((y.real.double() ** 2 + y.imag.double() ** 2).sum())
+    assert abs(ey / (N * ex) - 1) < (1e-5 if dt == "float2" else 1e-12)
+    x2 = torch.roll(x, 1, dims=0)                      # transform b of x2 is transform b-1 of x
+    y2 = plan.fft(x + x2)
+    torch.cuda.synchronize()
+    d = y2 - (y + torch.roll(y, 1, dims=0))
+    rel = float(d.abs().double().pow(2).sum().sqrt() / y2.abs().double().pow(2).sum().sqrt())
+    assert rel <= 2 * O.tolerance(dt, logN)
+
+
+def test_config3_full_size_fp64_2p15():
+    # BASELINE config 3 at full size: fp64, N=2^15, batch 2^13, standard normal input, two launches
+    plan = turbofft_amd.TurboFFT(15, "double2")
+    assert plan.launches == 2
+    _full_size_check(_torch(), plan, "double2", 15, 1 << 13, normal=True)
+
+
+def test_config4_full_size_fp32_2p24():
+    # BASELINE config 4 at full size: fp32, N=2^24, batch 16, three launches
+    plan = turbofft_amd.TurboFFT(24, "float2")
+    assert plan.launches == 3
+    _full_size_check(_torch(), plan, "float2", 24, 16, normal=False)
+
+
 def test_cli_verify_mode():
     for dt, logN, bs in ((1, 10, 16), (0, 13, 4), (1, 15, 2)):
         r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "0", "--if_verify", "1", "--logN", str(logN),
