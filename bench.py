@@ -78,7 +78,9 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
         "alg_bytes": plan.algorithmic_bytes(bs),
     }
     if if_ft or if_err:
+        # counters accumulate over every execution of the plan (warm-up included)
         res["ft"] = {k: v for k, v in plan.ft_counters().items() if k != "flagged"}
+        res["ft"]["execs"] = warmup + steps
     plan.close()
     return res, x, out
 
@@ -169,7 +171,9 @@ def main():
                     r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
                     print(f"{'fp32' if dt == 0 else 'fp64'} logN={logN:2d} L={r['launches']} "
                           f"{r['wall_ms']:8.3f} ms {r['gflops']:9.1f} GFLOPS {r['gbs']:8.1f} GB/s  "
-                          f"{100 * r['frac_hbm']:5.1f}% of HBM peak  {r['plan']}", flush=True)
+                          f"{100 * r['frac_hbm']:5.1f}% of HBM peak  {r['plan']}"
+                          + (f"  ft per exec: " + " ".join(f"{k} {v // r['ft']['execs']}" for k, v in r["ft"].items() if k != "execs")
+                             if "ft" in r else ""), flush=True)
                 else:
                     print(r, flush=True)
                 lines.append(r)
