@@ -264,3 +264,27 @@ def test_optional_kernel_variants(dt):
         assert c["detected"] == c["corrected"] > 0 and c["uncorrectable"] == 0
         for b in range(bs):
             assert O.rel_l2(yf[b], ref[b]) <= O.tolerance(dt, r.logN), (r, b, "ft")
+
+
+def test_seeded_random_shapes():
+    """Forty seeded draws of (type, logN, batch, tiles per block, fault tolerance): ragged
+    batches, every plan depth, plain and checksummed kernels, against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        dt = ["float2", "double2"][int(rng.integers(2))]
+        logN = int(rng.integers(1, 21))
+        bs = int(rng.integers(1, max(2, min(200, (1 << 22) >> logN))))
+        tbs = int(rng.choice([1, 1, 2, 3, 5, 8]))
+        ft = int(rng.integers(2))
+        plan = turbofft_amd.TurboFFT(logN, dt, if_ft=ft, thread_bs=tbs)
+        print(f"[random case {case}] ft={ft} thread_bs={tbs}", flush=True)
+        x = make(bs, 1 << logN, dt, 1000 + case, normal=bool(rng.integers(2)))
+        y = gpu_fft(plan, x)
+        ref = O.fft_ref(x)
+        assert O.rel_l2(y, ref) <= O.tolerance(dt, logN)
+        worst = max(O.rel_l2(y[b], ref[b]) for b in range(bs))
+        assert worst <= O.tolerance(dt, logN)
+        if ft:
+            c = plan.ft_counters()
+            assert c["detected"] == 0 and c["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
+        plan.close()
