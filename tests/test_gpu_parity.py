@@ -229,6 +229,22 @@ def test_cli_verify_mode():
         assert f"turboFFT, {logN}, " in r.stdout
 
 
+def test_cli_bench_modes():
+    # the reference's run scripts (compile.sh:12-29): --if_bench 2 prints one line per logN at
+    # logBS + logN = param_1; with FT the counters follow.  Restricted here to a few sizes.
+    for extra in ([], ["--if_ft", "1", "--if_err", "1", "--thread_bs", "4"]):
+        r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "2", "--datatype", "0", "--param_1", "22",
+                            "--logN_begin", "8", "--logN_end", "17"] + extra,
+                           capture_output=True, text=True, timeout=120)
+        print(r.stdout[-2000:], r.stderr[-500:], flush=True)
+        assert r.returncode == 0
+        lines = [ln for ln in r.stdout.splitlines() if ln.startswith("turboFFT, ")]
+        assert [int(ln.split(",")[1]) for ln in lines] == list(range(8, 18))
+        for ln in lines:                       # turboFFT, logN, logBS, ms, GFLOPS, GB/s
+            f = [v.strip() for v in ln.split(",")]
+            assert int(f[1]) + int(f[2]) == 22 and float(f[3]) > 0 and float(f[4]) > 0 and float(f[5]) > 0
+
+
 VARIANTS_DIR = os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param", "gfx950")
 
 

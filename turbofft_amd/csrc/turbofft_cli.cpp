@@ -57,6 +57,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
                   << "  --gpu <str>          Set GPU spec.\n"
                   << "  --param <file>       Plan CSV (default: built-in gfx950 table).\n"
                   << "  --logN_begin/--logN_end <value>  Restrict the --if_bench sweep.\n"
+                  << "  --param_1 <value>        logBS + logN of the --if_bench sweep (default 28; the reference derives it from --gpu).\n"
                   << "  -h, --help               Display this help message and exit.\n";
     }
 
@@ -76,6 +77,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
         else if (!strcmp(name, "--param")) param_file_path = value;
         else if (!strcmp(name, "--logN_begin")) logN_begin = atoi(value);
         else if (!strcmp(name, "--logN_end")) logN_end = atoi(value);
+        else if (!strcmp(name, "--param_1")) param_1 = atoi(value);
         else return false;
         return true;
     }
