@@ -199,7 +199,8 @@ extern "C" {
 const char* turbofft_last_error(void) { return g_err.c_str(); }
 
 int turbofft_build_twiddle_table(int datatype, long long N, void* out) {
-    if (!out || N < 1 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "twiddle table: N must be a power of two");
+    if (!out) return fail(TURBOFFT_EINVAL, "twiddle table: null output buffer");
+    if (N < 1 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "twiddle table: N must be a power of two");
     if (datatype == TURBOFFT_FP32) fill_twiddle((c32*)out, N);
     else if (datatype == TURBOFFT_FP64) fill_twiddle((c64*)out, N);
     else return fail(TURBOFFT_EINVAL, "bad datatype %d", datatype);
@@ -207,7 +208,8 @@ int turbofft_build_twiddle_table(int datatype, long long N, void* out) {
 }
 
 int turbofft_build_checksum_vector(int datatype, long long N, int mode, void* out) {
-    if (!out || N < 2 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "checksum vector: N must be a power of two >= 2");
+    if (!out) return fail(TURBOFFT_EINVAL, "checksum vector: null output buffer");
+    if (N < 2 || (N & (N - 1))) return fail(TURBOFFT_EINVAL, "checksum vector: N must be a power of two >= 2");
     if (datatype != TURBOFFT_FP32 && datatype != TURBOFFT_FP64) return fail(TURBOFFT_EINVAL, "bad datatype %d", datatype);
     if (mode == 1) {
         if (datatype == TURBOFFT_FP32) checksum_reference<c32, float>(N, (c32*)out);
