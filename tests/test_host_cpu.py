@@ -105,8 +105,15 @@ def test_checksum_vector_reference_mode_matches_oracle(dtype):
 
 def test_bad_arguments_are_reported_not_fatal():
     L = turbofft_amd.lib()
-    assert L.turbofft_build_twiddle_table(0, 3, None) != 0
+    buf = np.zeros(64, dtype=np.complex128)
+    assert L.turbofft_build_twiddle_table(0, 3, buf.ctypes.data) != 0
     assert b"power of two" in L.turbofft_last_error()
+    assert L.turbofft_build_twiddle_table(0, 8, None) != 0
+    assert b"null output" in L.turbofft_last_error()
+    assert L.turbofft_build_checksum_vector(1, 1, 0, buf.ctypes.data) != 0
+    assert b"power of two" in L.turbofft_last_error()
+    assert L.turbofft_build_checksum_vector(7, 8, 0, buf.ctypes.data) != 0
+    assert b"datatype" in L.turbofft_last_error()
     assert L.turbofft_exec(None, None, None, 1, None) != 0
     # plan creation needs a device: here it must fail with a message, not crash
     import torch
