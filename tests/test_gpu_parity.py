@@ -304,3 +304,33 @@ def test_seeded_random_shapes():
             c = plan.ft_counters()
             assert c["detected"] == 0 and c["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
         plan.close()
+
+
+@pytest.mark.parametrize("dt,logN,bs,ft", [("float2", 10, 7, 0), ("double2", 16, 3, 0), ("float2", 24, 1, 0), ("float2", 12, 9, 1)])
+def test_exec_inside_a_hip_graph(dt, logN, bs, ft):
+    """turbofft_exec allocates nothing and records no memset, so a plan can be captured into
+    a HIP graph; every replay (with new input written in between) must equal the eager result."""
+    torch = _torch()
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=ft, thread_bs=2 if ft else 1)
+    cdt = torch.complex64 if dt == "float2" else torch.complex128
+    x = torch.from_numpy(make(bs, 1 << logN, dt, 50)).cuda()
+    out = torch.empty(plan.out_elems(bs), dtype=cdt, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream.cuda_stream)        # warm-up outside the capture
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        x.copy_(torch.from_numpy(make(bs, 1 << logN, dt, 60 + rep)).cuda())
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out[: bs * (1 << logN)].view(bs, 1 << logN).clone()
+        eager = plan.fft(x).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep} differs from the eager run"
+        assert O.rel_l2(got.cpu().numpy(), O.fft_ref(x.cpu().numpy())) <= O.tolerance(dt, logN)
