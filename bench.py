@@ -11,6 +11,8 @@ whole batch.  Prints ONE JSON line:
                  events on the launch stream over the timed region
   cpu_baseline : scipy.fft (pocketfft) on the host cores for a bounded sample
                  of the same workload, scaled to the same unit
+  ft_overhead  : run time of the same workload with the fused checksums over the
+                 plain plan, measured after the timed region (--no_ft_overhead skips it)
 
 Other workloads for tuning: --logN/--datatype/--bs, --sweep (logN 7..24 at
 logBS+logN=28 for both types, one JSON line per case to --out).
@@ -133,6 +135,8 @@ def main():
     ap.add_argument("--sweep_lo", type=int, default=7)
     ap.add_argument("--sweep_hi", type=int, default=24)
     ap.add_argument("--out", type=str, default=None)
+    ap.add_argument("--no_ft_overhead", action="store_true",
+                    help="skip the extra fault-tolerant run that reports the FT overhead of the workload")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -191,6 +195,14 @@ def main():
     for _ in range(a.calib_copy):
         out.view(-1)[: x.numel()].copy_(x.view(-1))          # reads and writes x.numel()*sizeof(T) bytes
     torch.cuda.synchronize()
+    ft_line = None
+    if not (a.if_ft or a.if_err) and not a.no_ft_overhead:
+        # the second half of the headline metric: the same workload with the fused checksums
+        # (4 tiles per checksum group, no error injected), outside the timed region above
+        rf, x, out = run_case(torch, turbofft_amd, logN, dt, bs, max(20, a.steps // 4), min(a.warmup, 5), 1, 0, 4,
+                              a.param, x, out)
+        ft_line = {"overhead_pct": 100.0 * (rf["event_ms"] / r["event_ms"] - 1.0), "ms_per_step": rf["wall_ms"],
+                   "thread_bs": 4, "plan": rf["plan"], "counters": rf.get("ft")}
     del x, out
     tname = "fp32" if dt == 0 else "fp64"
     launches = r["launches"]
@@ -215,6 +227,8 @@ def main():
     }
     if a.if_ft or a.if_err:
         line["ft"] = r.get("ft")
+    if ft_line is not None:
+        line["ft_overhead"] = ft_line
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(logN, dt, a.cpu_seconds)
     print(json.dumps(line), flush=True)
