@@ -249,3 +249,52 @@ def test_injection_element_is_validated():
         plan.set_injection(2, every=1 << 30, tile_phase=0, s=0, m=lim)
     with pytest.raises(turbofft_amd.TurboFFTError):
         plan.set_injection(2, every=1 << 30, tile_phase=0, s=plan.BS[-1], m=0)
+
+
+def test_seeded_random_injections_match_the_model():
+    """Sixty seeded draws of (type, size, batch, group size, interleave, launch, element,
+    magnitude, cadence, correction on/off) with at most one error per checksum group: the
+    flagged (launch, tile) list and the counters equal the oracle model's decisions.  Draws
+    whose ratio sits within a factor 1.5 of the threshold are redrawn (reduction order
+    differs between the GPU and the model)."""
+    torch = _torch()
+    rng = np.random.default_rng(31)
+    done = 0
+    while done < 60:
+        dt = ["float2", "double2"][int(rng.integers(2))]
+        logN = int(rng.integers(4, 17))
+        tbs = int(rng.choice([1, 2, 3, 4, 8]))
+        plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=tbs)
+        row = O.PlanRow.from_list(plan.plan_row())
+        L = plan.launches
+        li = int(rng.integers(L))
+        bs = int(rng.integers(1, 7)) * plan.BS[0] * tbs if L == 1 else int(rng.integers(1, 1 + max(1, (1 << 20) >> logN)))
+        gaps = [int(rng.integers(1, 9)) for _ in range(L)]
+        for i, g in enumerate(gaps):
+            plan.set_tb_gap(i, g)
+        x = make(bs, 1 << logN, dt, 500 + done)
+        ntiles = O.launch_geometry(row, bs)[li].ntiles
+        every = (tbs - 1) * gaps[li] + 1 + int(rng.integers(0, 5))         # at most one error per group
+        phase = int(rng.integers(every))
+        s = int(rng.integers(plan.BS[li]))
+        m = int(rng.integers((1 << plan.logNi[li]) // plan.n[li]))
+        mag = float(10 ** rng.uniform(0, 5))
+        correct = bool(rng.integers(2))
+        injs = [O.Injection(t, s, m, mag) for t in range(phase, ntiles, every)]
+        dec, _ = O.ft_plan_model(x, row, dt, tbs, gaps, injs, inj_launch=li)
+        if any(0.67 <= abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3 <= 1.5 for dl in dec for d in dl):
+            plan.close()
+            continue
+        plan.set_ft_params(1000.0, 1e-3, correct=correct)
+        plan.set_injection(2, launch=li, every=every, tile_phase=phase, s=s, m=m, mag=mag)
+        print(f"[random injection {done}] launch={li} every={every} phase={phase} s={s} m={m} mag={mag:.1f} correct={correct} gaps={gaps}", flush=True)
+        y, c = run(plan, x)
+        model = sorted((l, d.tile) for l, dl in enumerate(dec) for d in dl if d.detected)
+        assert sorted(c["flagged"]) == model
+        assert c["detected"] == len(model) and c["uncorrectable"] == 0
+        assert c["corrected"] == (len(model) if correct else 0)
+        assert c["checked"] == sum(plan.grid(i, bs) for i in range(L))
+        if correct and len(model) == len(injs):          # every error caught and recomputed
+            assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+        plan.close()
+        done += 1
