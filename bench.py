@@ -13,9 +13,13 @@ whole batch.  Prints ONE JSON line:
                  of the same workload, scaled to the same unit
   ft_overhead  : run time of the same workload with the fused checksums over the
                  plain plan, measured after the timed region (--no_ft_overhead skips it)
+  vendor_baseline : hipFFT (rocFFT) on the same buffers and workload, after the timed
+                 region, the side-by-side the reference runs against cuFFT
+                 (main.cu:105,121); --no_vendor skips it
 
 Other workloads for tuning: --logN/--datatype/--bs, --sweep (logN 7..24 at
-logBS+logN=28 for both types, one JSON line per case to --out).
+logBS+logN=28 for both types, one JSON line per case to --out; with --vendor
+every case is followed by hipFFT on the same buffers).
 """
 import argparse
 import json
@@ -87,6 +91,21 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
     return res, x, out
 
 
+def vendor_case(torch, turbofft_amd, logN, datatype, bs, x, out, reps=20, warmup=2):
+    """hipFFT on the same device buffers; reported beside the result, never part of it."""
+    if not turbofft_amd.vendor_available():
+        return {"library": "hipFFT", "error": "libhipfft.so could not be opened"}
+    esize = 8 if datatype == 0 else 16
+    try:
+        ms = turbofft_amd.vendor_time(logN, datatype, x.data_ptr(), out.data_ptr(), bs, warmup, reps,
+                                      torch.cuda.current_stream().cuda_stream)
+    except turbofft_amd.TurboFFTError as e:
+        return {"library": "hipFFT", "error": str(e)}
+    pts = bs * (1 << logN)
+    return {"library": "hipFFT", "value": 2 * pts * esize / ms / 1e6, "unit": "GB/s", "ms_per_step": ms,
+            "gflops": 5.0 * pts * logN / ms / 1e6, "reps": reps}
+
+
 def cpu_baseline(logN, datatype, target_s=10.0):
     """Reference CPU path: pocketfft via scipy.fft on all host cores the box
     gives one GPU (16), on a bounded sample of the workload."""
@@ -137,6 +156,8 @@ def main():
     ap.add_argument("--out", type=str, default=None)
     ap.add_argument("--no_ft_overhead", action="store_true",
                     help="skip the extra fault-tolerant run that reports the FT overhead of the workload")
+    ap.add_argument("--no_vendor", action="store_true", help="skip the hipFFT side-by-side of the default line")
+    ap.add_argument("--vendor", action="store_true", help="--sweep: run hipFFT after every case")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -180,6 +201,14 @@ def main():
                              if "ft" in r else ""), flush=True)
                 else:
                     print(r, flush=True)
+                if a.vendor and "gbs" in r:
+                    v = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(5, a.steps // 4))
+                    r["vendor"] = v
+                    if "value" in v:
+                        print(f"     hipFFT      {v['ms_per_step']:8.3f} ms {v['gflops']:9.1f} GFLOPS {v['value']:8.1f} GB/s  "
+                              f"this library / hipFFT = {r['gbs'] / v['value']:.2f}", flush=True)
+                    else:
+                        print(f"     hipFFT      {v['error']}", flush=True)
                 lines.append(r)
             del x, out
             torch.cuda.empty_cache()
@@ -203,6 +232,9 @@ def main():
                               a.param, x, out)
         ft_line = {"overhead_pct": 100.0 * (rf["event_ms"] / r["event_ms"] - 1.0), "ms_per_step": rf["wall_ms"],
                    "thread_bs": 4, "plan": rf["plan"], "counters": rf.get("ft")}
+    vendor_line = None
+    if not a.no_vendor:
+        vendor_line = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(10, a.steps // 10))
     del x, out
     tname = "fp32" if dt == 0 else "fp64"
     launches = r["launches"]
@@ -229,6 +261,8 @@ def main():
         line["ft"] = r.get("ft")
     if ft_line is not None:
         line["ft_overhead"] = ft_line
+    if vendor_line is not None:
+        line["vendor_baseline"] = vendor_line
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(logN, dt, a.cpu_seconds)
     print(json.dumps(line), flush=True)

@@ -149,6 +149,27 @@ int turbofft_builtin_plan_row(int datatype, int logN, int row[11]);
 int turbofft_kernel_count(void);
 const char* turbofft_kernel_name(int i);
 
+/* ---- vendor-library side-by-side (measurement and cross-check only) ----
+ * The role of profiler::cufft::test_cufft (include/cufft/cufft.h:14-56 fp32,
+ * :59-101 fp64; called at main.cu:99,105,121) with hipFFT where the reference
+ * uses cuFFT.  hipFFT is opened with dlopen at first use; when it is absent
+ * these return TURBOFFT_ENOPLAN and the rest of the library is unaffected.
+ * No transform of this library is computed by the vendor code. */
+
+/* 1 when libhipfft.so can be opened, else 0. */
+int turbofft_vendor_available(void);
+
+/* One forward C2C/Z2Z transform of `bs` length-2^logN sequences by hipFFT,
+ * device pointers, synchronised on return (hipfftPlan1d + exec + destroy,
+ * cufft.h:23-31,48-52). */
+int turbofft_vendor_exec(int logN, int datatype, const void* in_d, void* out_d, long long bs, void* stream);
+
+/* Timed like turbofft_time: `warmup` untimed and `reps` timed executions of one
+ * hipFFT plan between two HIP events, no host synchronisation in between
+ * (cufft.h:26-42 synchronises after every execution). */
+int turbofft_vendor_time(int logN, int datatype, const void* in_d, void* out_d, long long bs,
+                         int warmup, int reps, void* stream, float* ms_per_exec);
+
 /* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
  * flags and output lines.  Returns the process exit code. */
 int turbofft_main(int argc, char** argv);

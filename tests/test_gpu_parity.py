@@ -229,6 +229,48 @@ def test_cli_verify_mode():
         assert f"turboFFT, {logN}, " in r.stdout
 
 
+@pytest.mark.parametrize("dt,logN,bs", [("double2", 10, 16), ("float2", 13, 64), ("double2", 15, 8),
+                                        ("float2", 20, 4), ("float2", 24, 1)])
+def test_agrees_with_the_vendor_library(dt, logN, bs):
+    # the reference's own check (main.cu:98-102): its result against the vendor library's on the
+    # same device input.  Both are roundings of the same transform, so they differ by at most the
+    # sum of their error bounds.
+    torch = _torch()
+    if not turbofft_amd.vendor_available():
+        pytest.skip("libhipfft.so cannot be opened")
+    N = 1 << logN
+    x = torch.view_as_complex(torch.rand((bs, N, 2), generator=torch.Generator(device="cuda").manual_seed(logN),
+                                         device="cuda", dtype=torch.float32 if dt == "float2" else torch.float64) * 2 - 1)
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    ours = plan.fft(x).clone()
+    theirs = turbofft_amd.vendor_fft(x)
+    err = (torch.linalg.vector_norm(ours - theirs) / torch.linalg.vector_norm(theirs)).item()
+    tol = 2 * (1e-5 if dt == "float2" else 1e-13) * logN
+    print(f"{dt} logN={logN} bs={bs}: rel L2 difference to hipFFT {err:.3e} (tol {tol:.1e})", flush=True)
+    assert err <= tol
+    plan.close()
+
+
+def test_cli_vendor_modes():
+    # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
+    # comparison with its result after the one with the host FFT
+    if not turbofft_amd.vendor_available():
+        pytest.skip("libhipfft.so cannot be opened")
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "12", "--datatype", "0", "--param_1", "22",
+                        "--logN_begin", "9", "--logN_end", "12"], capture_output=True, text=True, timeout=300)
+    print(r.stdout[-2000:], r.stderr[-500:], flush=True)
+    assert r.returncode == 0
+    lines = [ln for ln in r.stdout.splitlines() if ln.startswith("hipFFT, ")]
+    assert [int(ln.split(",")[1]) for ln in lines] == [9, 10, 11, 12]
+    assert not [ln for ln in r.stdout.splitlines() if ln.startswith("turboFFT, ")]
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "0", "--if_verify", "1", "--if_profile", "1", "--logN", "12",
+                        "--bs", "8", "--bs_end", "8", "--datatype", "1"], capture_output=True, text=True, timeout=300)
+    print(r.stdout[-2000:], r.stderr[-500:], flush=True)
+    assert r.returncode == 0 and "Error detected" not in r.stdout
+    assert r.stdout.count("Compare finished.") == 2
+    assert r.stdout.count("hipFFT, 12, 3,") == 2 and r.stdout.count("turboFFT, 12, 3,") == 2
+
+
 def test_cli_bench_modes():
     # the reference's run scripts (compile.sh:12-29): --if_bench 2 prints one line per logN at
     # logBS + logN = param_1; with FT the counters follow.  Restricted here to a few sizes.

@@ -122,6 +122,16 @@ def test_bad_arguments_are_reported_not_fatal():
             turbofft_amd.TurboFFT(10, "double2")
 
 
+def test_vendor_side_by_side_rejects_bad_arguments_before_touching_a_device():
+    L = turbofft_amd.lib()
+    ms = ctypes.c_float(0)
+    assert L.turbofft_vendor_exec(10, 0, None, None, 4, None) != 0
+    assert b"null buffer" in L.turbofft_last_error()
+    assert L.turbofft_vendor_time(10, 0, None, None, 4, 1, 10, None, ctypes.byref(ms)) != 0
+    assert b"bad argument" in L.turbofft_last_error()
+    assert turbofft_amd.vendor_available() in (True, False)      # opening the library needs no device
+
+
 def test_cli_help_and_bad_flag():
     import subprocess
     r = subprocess.run([turbofft_amd.CLI_PATH, "--help"], capture_output=True, text=True)

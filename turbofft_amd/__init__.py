@@ -78,6 +78,8 @@ def lib() -> C.CDLL:
     L.turbofft_kernel_name.restype = C.c_char_p
     L.turbofft_kernel_name.argtypes = [i]
     L.turbofft_main.argtypes = [i, C.POINTER(C.c_char_p)]
+    L.turbofft_vendor_exec.argtypes = [i, i, vp, vp, ll, vp]
+    L.turbofft_vendor_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     _lib = L
     return L
 
@@ -111,6 +113,34 @@ def builtin_plan_row(datatype, logN: int) -> List[int]:
 def kernel_names() -> List[str]:
     L = lib()
     return [L.turbofft_kernel_name(i).decode() for i in range(L.turbofft_kernel_count())]
+
+
+# ---- vendor-library side-by-side (hipFFT; the role of cufft/cufft.h in the reference) ----
+def vendor_available() -> bool:
+    return bool(lib().turbofft_vendor_available())
+
+
+def vendor_fft(x, out=None):
+    """hipFFT forward transform of a (bs, N) complex tensor on the GPU; measurement and
+    cross-check only (main.cu:99-101 compares the reference's result with cuFFT's)."""
+    import torch
+    if x.dim() != 2 or not x.is_cuda or not x.is_contiguous() or x.dtype not in (torch.complex64, torch.complex128):
+        raise ValueError("expected a contiguous complex64/complex128 tensor of shape (bs, N) on the GPU")
+    bs, N = x.shape
+    logN = N.bit_length() - 1
+    if N != 1 << logN:
+        raise ValueError("N must be a power of two")
+    if out is None:
+        out = torch.empty_like(x)
+    _check(lib().turbofft_vendor_exec(logN, FP32 if x.dtype == torch.complex64 else FP64, x.data_ptr(), out.data_ptr(), bs,
+                                      torch.cuda.current_stream(x.device).cuda_stream))
+    return out
+
+
+def vendor_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0) -> float:
+    ms = C.c_float(0)
+    _check(lib().turbofft_vendor_time(logN, _datatype(datatype), in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
+    return ms.value
 
 
 def turbofft_main(argv: List[str]) -> int:

@@ -5,11 +5,14 @@
 //        (compareData.h:4-35, tolerance 1e-4).  The reference compares with
 //        cuFFT (main.cu:98-102); here the comparison values come from a plain
 //        fp64 radix-2 FFT on the host that exists only for this check and is
-//        never used to produce results.
-//   --if_profile 1 --if_bench 0                  timed runs for bs..bs_end step bs_gap
+//        never used to produce results, and then, when hipFFT can be opened,
+//        from hipFFT on the same device buffers as well.
+//   --if_profile 1 --if_bench 0                  timed runs for bs..bs_end step bs_gap,
+//                                                hipFFT first when present (main.cu:104-110)
 //   --if_bench 1                                 logN = 1..25, bs = 1..2^(28-logN)
 //   --if_bench 2                                 logN = 1..25, bs = 2^(28-logN)
-//   --if_bench 11/12                             (cuFFT baseline in the reference) not built
+//   --if_bench 11/12                             the same two sweeps with hipFFT (cuFFT in the
+//                                                reference, main.cu:121)
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -48,8 +51,8 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
                   << "  --if_verify <0|1>    Enable (1) or disable (0) verification.\n"
                   << "  --if_bench <0|1|2|11|12> Enable (1) or disable (0) benchmarking.\n"
                   << "                           (2) for logBS + logN = 28.\n"
-                  << "                           (11) for the vendor FFT library (not built).\n"
-                  << "                           (12) for the vendor FFT library & logBS + logN = 28 (not built).\n"
+                  << "                           (11) for hipFFT.\n"
+                  << "                           (12) for hipFFT & logBS + logN = 28.\n"
                   << "  --if_ft <0|1>        Enable (1) or disable (0) fault tolerance.\n"
                   << "  --if_err <0|1>       Enable (1) or disable (0) error injection.\n"
                   << "  --datatype <type>    0 for FP32, 1 for FP64.\n"
@@ -210,6 +213,22 @@ int test_turbofft(const ProgramConfig& cfg, int logN, long long bs, int ntest, B
     return rc;
 }
 
+// test_cufft (cufft/cufft.h:14-56): the vendor library on the same buffers, same metric line
+int test_vendor_fft(const ProgramConfig& cfg, int logN, long long bs, int ntest, Buffers& b, std::vector<char>* result) {
+    float ms = 0;
+    int rc = turbofft_vendor_time(logN, cfg.datatype, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms);
+    if (rc) { printf("hipFFT, %d: %s\n", logN, turbofft_last_error()); return rc; }
+    double N = (double)(1ll << logN);
+    double gflops = 5.0 * N * logN * (double)bs / ms * 1000.0 / 1e9;             // cufft.h:41
+    double gbs = N * (double)bs * (double)b.esize * 2.0 / ms * 1000.0 / 1e9;     // cufft.h:44
+    printf("hipFFT, %d, %d, %8.3f, %8.3f, %8.3f\n", logN, (int)log2((double)bs), ms, gflops, gbs);
+    if (result) {
+        result->resize((size_t)(1ll << logN) * bs * b.esize);
+        if (hipMemcpy(result->data(), b.out_d, result->size(), hipMemcpyDeviceToHost) != hipSuccess) rc = -1;   // cufft.h:46-47
+    }
+    return rc;
+}
+
 }  // namespace
 
 extern "C" int turbofft_main(int argc, char** argv) {
@@ -218,13 +237,14 @@ extern "C" int turbofft_main(int argc, char** argv) {
     if (pc) return pc - 1;
     cfg.displayConfig();
     const int ntest = 10;
-    if (cfg.if_bench > 10) {
-        printf("--if_bench %d selects the vendor-library baseline, which this build does not include.\n", cfg.if_bench);
-        return EXIT_FAILURE;
-    }
     int dev_count = 0;
     if (hipGetDeviceCount(&dev_count) != hipSuccess || dev_count < 1) {
         printf("no HIP device available\n");
+        return EXIT_FAILURE;
+    }
+    const bool vendor = turbofft_vendor_available();
+    if (cfg.if_bench > 10 && !vendor) {
+        printf("--if_bench %d selects hipFFT, which could not be opened (libhipfft.so).\n", cfg.if_bench);
         return EXIT_FAILURE;
     }
     if (!cfg.if_bench) {
@@ -248,10 +268,25 @@ extern "C" int turbofft_main(int argc, char** argv) {
             }
             if (cfg.datatype == 0) compareData((const float*)res.data(), ref, cfg.N * cfg.bs, 1e-4);
             else compareData((const double*)res.data(), ref, cfg.N * cfg.bs, 1e-4);
+            if (vendor) {                       // main.cu:99-101: the same comparison with the vendor library's result
+                std::vector<char> vres;
+                if (test_vendor_fft(cfg, (int)cfg.logN, cfg.bs, 1, b, &vres)) return EXIT_FAILURE;
+                for (size_t i = 0; i < ref.size(); ++i)
+                    ref[i] = cfg.datatype == 0 ? std::complex<double>(((float*)vres.data())[2 * i], ((float*)vres.data())[2 * i + 1])
+                                               : std::complex<double>(((double*)vres.data())[2 * i], ((double*)vres.data())[2 * i + 1]);
+                if (cfg.datatype == 0) compareData((const float*)res.data(), ref, cfg.N * cfg.bs, 1e-4);
+                else compareData((const double*)res.data(), ref, cfg.N * cfg.bs, 1e-4);
+            } else {
+                printf("hipFFT could not be opened: compared with the host FFT only.\n");
+            }
         }
-        if (cfg.if_profile)
+        if (cfg.if_profile) {
+            if (vendor)
+                for (long long bs = cfg.bs; bs <= std::max(cfg.bs, cfg.bs_end); bs += cfg.bs_gap)
+                    if (test_vendor_fft(cfg, (int)cfg.logN, bs, ntest, b, nullptr)) return EXIT_FAILURE;
             for (long long bs = cfg.bs; bs <= std::max(cfg.bs, cfg.bs_end); bs += cfg.bs_gap)
                 if (test_turbofft(cfg, (int)cfg.logN, bs, ntest, b, nullptr)) return EXIT_FAILURE;
+        }
         return 0;
     }
     // benchmark sweep (main.cu:114-128)
@@ -261,7 +296,8 @@ extern "C" int turbofft_main(int argc, char** argv) {
         long long bs = 1;
         if (cfg.if_bench % 10 == 2) bs <<= (cfg.param_1 - logN);
         for (int i = 0; i <= cfg.param_1 - logN; ++i) {
-            test_turbofft(cfg, logN, bs, ntest, b, nullptr);
+            if (cfg.if_bench > 10) test_vendor_fft(cfg, logN, bs, ntest, b, nullptr);
+            else test_turbofft(cfg, logN, bs, ntest, b, nullptr);
             bs *= 2;
             if (cfg.if_bench % 10 == 2) break;
         }
