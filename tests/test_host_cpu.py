@@ -61,7 +61,8 @@ def test_builtin_rows_match_csv_and_are_consistent(dtype):
 
 def test_optional_plan_columns():
     """Columns beyond the reference's 11: per-launch split / prefetch / cross-lane flags,
-    tiles per block, per-launch wavefronts per SIMD.  Shorter rows mean zeros."""
+    tiles per block, per-launch wavefronts per SIMD, per-launch non-temporal accesses.
+    Shorter rows mean zeros."""
     from turbofft_amd.codegen.fft_codegen import generate_source
     r = P.PlanRow.from_list([19, 2, 9, 10, 0, 32, 16, 0, 32, 32, 0, 1, 1, 0, 0, 0, 0, 0, 0, 0, 8, 4, 3])
     assert (r.split, r.pf, r.xl, r.tiles, r.wv) == ((1, 1), (0, 0), (0, 0), 8, (4, 3))
@@ -71,6 +72,15 @@ def test_optional_plan_columns():
     assert [k.name for k in P.kernels_for_row(r, "float2", 1)] == ["tfft_f32_col_N9_b32_n32_s_ft", "tfft_f32_rowT_N10_b16_n32_s_ft"]
     src = generate_source([KernelSpec(plain[0])], False)
     assert "amdgpu_waves_per_eu(4, 4)" in src
+    # columns 25-27: non-temporal tile loads (1), stores (2) or both (3), for both flavours
+    r = P.PlanRow.from_list([19, 2, 9, 10, 0, 32, 16, 0, 32, 32, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 3, 2])
+    assert r.nt == (3, 2)
+    assert [k.name for k in P.kernels_for_row(r, "float2", 0)] == ["tfft_f32_col_N9_b32_n32_t3", "tfft_f32_rowT_N10_b16_n32_t2"]
+    assert [k.name for k in P.kernels_for_row(r, "float2", 1)] == ["tfft_f32_col_N9_b32_n32_t3_ft", "tfft_f32_rowT_N10_b16_n32_t2_ft"]
+    src = generate_source([KernelSpec(P.kernels_for_row(r, "float2", 0)[1])], False)
+    assert "GLDG(" in src and "GSTGN(" in src and "GLDGN(" not in src and "GSTG(" not in src
+    with pytest.raises(ValueError):
+        P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0] + [0] * 13 + [4])
     short = P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0])
     assert (short.split, short.tiles, short.wv) == ((0,), 0, (0,))
     assert "amdgpu_waves_per_eu" not in generate_source([KernelSpec(P.kernels_for_row(short, "float2", 0)[0])], False)

@@ -187,6 +187,13 @@ class KernelEmitter:
         # transposing kernels measured 1-9 % slower that way and keep plain global pointers.
         buf = spec.kind == "row1"
         self.GLD, self.GST = ("GLDU", "GSTU") if buf else ("GLDG", "GSTG")
+        # Non-temporal variants for the tile data only (it is touched once); twiddles and the
+        # checksum table are re-read by every tile and stay on the cached path.
+        nt = int(spec.key.nt)
+        if nt & 1:
+            self.GLD += "N"
+        if nt & 2:
+            self.GST += "N"
         self.TWL, self.TWLU = ("TWLD", "TWLDU") if buf else ("TWLG", "TWLGU")
 
     # ---------- literals ----------
@@ -935,7 +942,7 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     kinds = {"row1": 0, "col": 1, "rowT": 2}
     for sp in specs:
         k = sp.key
-        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {int(k.wv)}, {sp.threads}, {sp.lds_bytes}}},')
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {int(k.wv)}, {int(k.nt)}, {sp.threads}, {sp.lds_bytes}}},')
     c("};")
     c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")

@@ -10,7 +10,9 @@ rounds), three more `p1, p2, p3` the next-tile prefetch and three more
 21st column is the number of tiles a block of a plain (not fault-tolerant) plan
 walks when the caller leaves thread_bs at 1 (0 or absent: one); columns 22-24
 `w1, w2, w3` ask the compiler to fit that many wavefronts per SIMD (0: its own
-choice) for the plain kernel of the launch.  Launch i transforms a digit of size 2^logNi with BSi
+choice) for the plain kernel of the launch; columns 25-27 `t1, t2, t3` mark the
+launch's tile loads (1), stores (2) or both (3) as non-temporal (streamed past the
+caches; tables and twiddles stay cached).  Launch i transforms a digit of size 2^logNi with BSi
 sub-FFTs per tile and ni elements per thread; launch 0 owns the most-strided
 digit and the last launch the contiguous one.
 """
@@ -32,6 +34,7 @@ class PlanRow:
     xl: Tuple[int, ...] = ()         # optional columns 18-20: 1 = last small-radix pass across lanes
     tiles: int = 0                   # optional column 21: tiles per block of the plain plan (0 = 1)
     wv: Tuple[int, ...] = ()         # optional columns 22-24: wavefronts per SIMD to compile for (0 = free)
+    nt: Tuple[int, ...] = ()         # optional columns 25-27: 1 = non-temporal tile loads, 2 = stores, 3 = both
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -46,7 +49,9 @@ class PlanRow:
         ext3 = (row[17:20] + [0, 0, 0])[:3]
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
                     tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
-                    tuple((row[21:24] + [0, 0, 0])[:L]))
+                    tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]))
+        if any(t not in (0, 1, 2, 3) for t in p.nt):
+            raise ValueError(f"non-temporal columns must be 0..3 in row {row}")
         if L and sum(p.logNi) != p.logN:
             raise ValueError(f"logN1+logN2+logN3 != logN in row {row}")
         return p
@@ -68,12 +73,13 @@ class KernelKey:
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
     wv: int = 0      # > 0: compiled to fit this many wavefronts per SIMD (register budget 512 / wv)
+    nt: int = 0      # bit 0: tile loads are non-temporal, bit 1: tile stores are
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + ("_ft" if self.ft else ""))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_ft" if self.ft else ""))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:
@@ -83,7 +89,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:24] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:27] if t.strip()]))
     return rows
 
 
@@ -97,8 +103,10 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
                       # fault-tolerant plans keep the LDS path: the checksum model fixes which
                       # outputs a thread owns
                       (int(row.xl[i]) if row.xl else 0) if not ft else 0,
-                      # the register budget hint was tuned on the plain kernel only
-                      (int(row.wv[i]) if row.wv else 0) if not ft else 0)
+                      # the register budget hint was tuned on the plain kernel only (fault-tolerant
+                      # kernels keep their table in registers and spill under any tighter budget)
+                      (int(row.wv[i]) if row.wv else 0) if not ft else 0,
+                      int(row.nt[i]) if row.nt else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 
 

@@ -24,34 +24,59 @@ typedef unsigned tfft_u4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t tfft_rsrc(const void* p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, -1, 0x00020000);
 }
+// AUX is the cache-policy immediate of the instruction: 0 = default, 2 = non-temporal (nt)
+template <int AUX = 0>
 __device__ __forceinline__ float2 tfft_bld(const float2* p, unsigned voff, unsigned soff) {
-    const tfft_u2 t = __builtin_amdgcn_raw_buffer_load_b64(tfft_rsrc(p), voff, soff, 0);
+    const tfft_u2 t = __builtin_amdgcn_raw_buffer_load_b64(tfft_rsrc(p), voff, soff, AUX);
     float2 r; r.x = __uint_as_float(t.x); r.y = __uint_as_float(t.y); return r;
 }
+template <int AUX = 0>
 __device__ __forceinline__ double2 tfft_bld(const double2* p, unsigned voff, unsigned soff) {
-    const tfft_u4 t = __builtin_amdgcn_raw_buffer_load_b128(tfft_rsrc(p), voff, soff, 0);
+    const tfft_u4 t = __builtin_amdgcn_raw_buffer_load_b128(tfft_rsrc(p), voff, soff, AUX);
     double2 r; r.x = __hiloint2double((int)t.y, (int)t.x); r.y = __hiloint2double((int)t.w, (int)t.z); return r;
 }
+template <int AUX = 0>
 __device__ __forceinline__ void tfft_bst(float2* p, unsigned voff, unsigned soff, float2 v) {
     tfft_u2 t; t.x = __float_as_uint(v.x); t.y = __float_as_uint(v.y);
-    __builtin_amdgcn_raw_buffer_store_b64(t, tfft_rsrc(p), voff, soff, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(t, tfft_rsrc(p), voff, soff, AUX);
 }
+template <int AUX = 0>
 __device__ __forceinline__ void tfft_bst(double2* p, unsigned voff, unsigned soff, double2 v) {
     tfft_u4 t;
     t.x = (unsigned)__double2loint(v.x); t.y = (unsigned)__double2hiint(v.x);
     t.z = (unsigned)__double2loint(v.y); t.w = (unsigned)__double2hiint(v.y);
-    __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, AUX);
 }
 #define TFFT_ESZ(p) ((unsigned)sizeof(*(p)))
-#define GLDU(p, ub, uo, off) tfft_bld((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
-#define GSTU(p, ub, uo, off, v) tfft_bst((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
+#define GLDU(p, ub, uo, off) tfft_bld<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
+#define GSTU(p, ub, uo, off, v) tfft_bst<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
+// the same accesses marked non-temporal: tile data is touched once, so it need not displace
+// the tables in the caches
+#define GLDUN(p, ub, uo, off) tfft_bld<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
+#define GSTUN(p, ub, uo, off, v) tfft_bst<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
 // plain global-pointer forms of the same accesses
 #define GLDG(p, ub, uo, off) (((p) + ((ub) + (uo)))[(off)])
 #define GSTG(p, ub, uo, off, v) (((p) + ((ub) + (uo)))[(off)] = (v))
+typedef float tfft_f2v __attribute__((ext_vector_type(2)));
+typedef double tfft_d2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float2 tfft_gldn(const float2* p) {
+    const tfft_f2v t = __builtin_nontemporal_load((const tfft_f2v*)p); float2 r; r.x = t.x; r.y = t.y; return r;
+}
+__device__ __forceinline__ double2 tfft_gldn(const double2* p) {
+    const tfft_d2v t = __builtin_nontemporal_load((const tfft_d2v*)p); double2 r; r.x = t.x; r.y = t.y; return r;
+}
+__device__ __forceinline__ void tfft_gstn(float2* p, float2 v) {
+    tfft_f2v t; t.x = v.x; t.y = v.y; __builtin_nontemporal_store(t, (tfft_f2v*)p);
+}
+__device__ __forceinline__ void tfft_gstn(double2* p, double2 v) {
+    tfft_d2v t; t.x = v.x; t.y = v.y; __builtin_nontemporal_store(t, (tfft_d2v*)p);
+}
+#define GLDGN(p, ub, uo, off) tfft_gldn(((p) + ((ub) + (uo))) + (off))
+#define GSTGN(p, ub, uo, off, v) tfft_gstn(((p) + ((ub) + (uo))) + (off), (v))
 #define TWLG(p, i) ((p)[(i)])
 #define TWLGU(p, c, i) ((p)[(c) + (i)])
-#define TWLD(p, i) tfft_bld((p), (unsigned)(i) * TFFT_ESZ(p), 0u)
-#define TWLDU(p, c, i) tfft_bld((p), (unsigned)(i) * TFFT_ESZ(p), (unsigned)(c) * TFFT_ESZ(p))
+#define TWLD(p, i) tfft_bld<0>((p), (unsigned)(i) * TFFT_ESZ(p), 0u)
+#define TWLDU(p, c, i) tfft_bld<0>((p), (unsigned)(i) * TFFT_ESZ(p), (unsigned)(c) * TFFT_ESZ(p))
 #define LLD(i) (lds[(i)])
 #define LST(i, v) (lds[(i)] = (v))
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
@@ -79,6 +104,10 @@ extern long long tfft_sim_errors;
 #define GSTU(p, ub, uo, off, v) ((p)[TFFT_CHK((long long)(ub) + (long long)(uo) + (long long)(off), p##_limit, #p)] = (v))
 #define GLDG(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTG(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
+#define GLDUN(p, ub, uo, off) GLDU(p, ub, uo, off)
+#define GSTUN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
+#define GLDGN(p, ub, uo, off) GLDU(p, ub, uo, off)
+#define GSTGN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
 #define TWLG(p, i) TWLD(p, i)
 #define TWLGU(p, c, i) TWLDU(p, c, i)
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])

@@ -62,9 +62,11 @@ constexpr double kPi = 3.14159265358979323846;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[24];           // 11 reference columns + optional per-launch flags: split exchange,
-                         // prefetch, cross-lane last pass; then the tiles-per-block hint and
-                         // the per-launch wavefronts-per-SIMD the kernel was compiled for
+    int v[27];           // 11 reference columns + optional per-launch flags: split exchange,
+                         // prefetch, cross-lane last pass; then the tiles-per-block hint, the
+                         // per-launch wavefronts-per-SIMD the plain kernel was compiled for and
+                         // the per-launch non-temporal access bits
+    int nt(int i) const { return v[24 + i]; }
     int tiles() const { return v[20]; }
     int wv(int i) const { return v[21 + i]; }
     int split(int i) const { return v[11 + i]; }
@@ -88,7 +90,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 24 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 27 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -100,12 +102,12 @@ int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
     return i == launches - 1 ? 2 : 1;
 }
 
-const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv) {
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv, int nt) {
     int cnt = 0;
     const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
-            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv)
+            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt)
             return &t[i];
     return nullptr;
 }
@@ -320,7 +322,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
         int kind = kind_of_launch(p->launches, i);
         const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
                                                  (r.xl(i) && !p->if_ft) ? 1 : 0,    // FT plans keep the LDS path
-                                                 p->if_ft ? 0 : r.wv(i));
+                                                 p->if_ft ? 0 : r.wv(i), r.nt(i));
         if (!k)
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
