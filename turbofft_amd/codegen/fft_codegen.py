@@ -532,10 +532,12 @@ class KernelEmitter:
         sp = self.s
         c("if (!is_redo) {")
         c.ind += 1
-        c(f"{self.R} acc = 0;")
+        # two independent multiply-add chains (one per component): two operations per element;
+        # a single `acc += a*b + c*d` costs three, since the sum may not be reassociated
+        c(f"{self.R} acc = 0, acy = 0;")
         if self.ft_table_resident():
             for e in range(sp.n):
-                c(f"acc += r[{e}].x * cvr[{e}].x + r[{e}].y * cvr[{e}].y;")
+                c(f"acc += r[{e}].x * cvr[{e}].x; acy += r[{e}].y * cvr[{e}].y;")
         else:
             # The table is fetched after the data in batches of 8 (a 1024-thread block leaves
             # 128 registers per lane), every load of a batch issued back to back and waited for
@@ -548,8 +550,9 @@ class KernelEmitter:
                     c(f"cv[{e - b0}] = {self.TWLU}(ck, {sp.Tr * e}u, xc);")
                 c("SCHED_FENCE();")
                 for e in range(b0, min(sp.n, b0 + B)):
-                    c(f"acc += r[{e}].x * cv[{e - b0}].x + r[{e}].y * cv[{e - b0}].y;")
+                    c(f"acc += r[{e}].x * cv[{e - b0}].x; acy += r[{e}].y * cv[{e - b0}].y;")
                 c("SCHED_FENCE();")
+        c("acc += acy;")
         c("fin1 += acc; fin2 += cntf * acc;")
         # the injected element is one of the first Ni/n of its sub-FFT (register 0 of thread
         # x = m; the reference injects at m = 0)
@@ -572,11 +575,12 @@ class KernelEmitter:
             sel = [pq[(v + cc) % 3] for v in range(3)]
             c(f"const {self.R} rp{cc} = (x3 == 0u) ? {self.lit(sel[0][0])} : ((x3 == 1u) ? {self.lit(sel[1][0])} : {self.lit(sel[2][0])});")
             c(f"const {self.R} rq{cc} = (x3 == 0u) ? {self.lit(sel[0][1])} : ((x3 == 1u) ? {self.lit(sel[1][1])} : {self.lit(sel[2][1])});")
-        c(f"{self.R} acc = 0;")
+        c(f"{self.R} acc = 0, acy = 0;")
         for e in range(sp.n):
             ce = (sp.Tr * e) % 3
             reg = self.out_reg(e)
-            c(f"acc += r[{reg}].x * rp{ce} + r[{reg}].y * rq{ce};")
+            c(f"acc += r[{reg}].x * rp{ce}; acy += r[{reg}].y * rq{ce};")
+        c("acc += acy;")
         c("fo1 -= acc; fo2 -= cntf * acc;")
         c.ind -= 1
         c("}")
