@@ -12,7 +12,9 @@ whole batch.  Prints ONE JSON line:
   cpu_baseline : scipy.fft (pocketfft) on the host cores for a bounded sample
                  of the same workload, scaled to the same unit
   ft_overhead  : run time of the same workload with the fused checksums over the
-                 plain plan, measured after the timed region (--no_ft_overhead skips it)
+                 plain plan, measured after the timed region (--no_ft_overhead skips it);
+                 "offline" inside it is the same comparison for separate checksum passes
+                 before and after the plain plan (the reference's cufft_ft.h baseline)
   vendor_baseline : hipFFT (rocFFT) on the same buffers and workload, after the timed
                  region, the side-by-side the reference runs against cuFFT
                  (main.cu:105,121); --no_vendor skips it
@@ -158,6 +160,7 @@ def main():
                     help="skip the extra fault-tolerant run that reports the FT overhead of the workload")
     ap.add_argument("--no_vendor", action="store_true", help="skip the hipFFT side-by-side of the default line")
     ap.add_argument("--vendor", action="store_true", help="--sweep: run hipFFT after every case")
+    ap.add_argument("--offline", action="store_true", help="--sweep: time the offline checksum scheme after every case")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -201,6 +204,11 @@ def main():
                              if "ft" in r else ""), flush=True)
                 else:
                     print(r, flush=True)
+                if a.offline and "gbs" in r:
+                    oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(5, a.steps // 4),
+                                                              torch.cuda.current_stream().cuda_stream)
+                    r["offline_ft"] = {"ms_per_step": oms, "flagged": oflag, "overhead_pct": 100.0 * (oms / r["event_ms"] - 1.0)}
+                    print(f"     offline FT  {oms:8.3f} ms  +{r['offline_ft']['overhead_pct']:.1f} % over the plain plan, {oflag} flagged", flush=True)
                 if a.vendor and "gbs" in r:
                     v = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(5, a.steps // 4))
                     r["vendor"] = v
@@ -232,6 +240,13 @@ def main():
                               a.param, x, out)
         ft_line = {"overhead_pct": 100.0 * (rf["event_ms"] / r["event_ms"] - 1.0), "ms_per_step": rf["wall_ms"],
                    "thread_bs": 4, "plan": rf["plan"], "counters": rf.get("ft")}
+        # the offline scheme on the same workload: checksum pass, plain plan, checksum pass, compare
+        try:
+            oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 10),
+                                                      torch.cuda.current_stream().cuda_stream)
+            ft_line["offline"] = {"overhead_pct": 100.0 * (oms / r["event_ms"] - 1.0), "ms_per_step": oms, "flagged": oflag}
+        except turbofft_amd.TurboFFTError as e:
+            ft_line["offline"] = {"error": str(e)}
     vendor_line = None
     if not a.no_vendor:
         vendor_line = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(10, a.steps // 10))

@@ -170,6 +170,28 @@ int turbofft_vendor_exec(int logN, int datatype, const void* in_d, void* out_d, 
 int turbofft_vendor_time(int logN, int datatype, const void* in_d, void* out_d, long long bs,
                          int warmup, int reps, void* stream, float* ms_per_exec);
 
+/* ---- offline checksums (measurement and cross-check only) ----
+ * The baseline the fused scheme is compared with (include/cufft/cufft_ft.h:19-95:
+ * checksum pass over the input, library transform, checksum pass over the output,
+ * each its own launch; the reference pairs cuBLAS gemv with cuFFT).  Same
+ * arithmetic as the fused kernels, per transform:
+ *   in_sums[b]  = re+im of sum_m x[b][m] c_N[m],   out_sums[b] = re+im of sum_k y[b][k] r[k%3]. */
+
+/* The two checksum passes alone, on a given input and an already computed
+ * output; in_sums_d / out_sums_d receive bs values of the real type (float or
+ * double) in device memory.  Synchronised on return. */
+int turbofft_offline_checksums(int logN, int datatype, const void* in_d, const void* out_d, long long bs,
+                               void* in_sums_d, void* out_sums_d, void* stream);
+
+/* Timed like turbofft_time: input pass, this library's plain plan, output pass
+ * and the per-transform comparison |in - out| / (1000 + mag) > 1e-3, `reps`
+ * times between two HIP events.  out_d as for turbofft_exec (2*N*bs elements
+ * when the plan has more than one launch).  *flagged_rows (may be NULL)
+ * receives the number of transforms the last repetition flagged. */
+int turbofft_offline_ft_time(int logN, int datatype, const void* in_d, void* out_d, long long bs,
+                             int warmup, int reps, void* stream, float* ms_per_exec,
+                             unsigned long long* flagged_rows);
+
 /* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
  * flags and output lines.  Returns the process exit code. */
 int turbofft_main(int argc, char** argv);

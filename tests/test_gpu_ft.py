@@ -298,3 +298,55 @@ def test_seeded_random_injections_match_the_model():
             assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
         plan.close()
         done += 1
+
+
+@pytest.mark.parametrize("dt,logN,bs", [("float2", 10, 64), ("double2", 13, 8), ("float2", 16, 4), ("double2", 7, 300),
+                                        ("float2", 1, 5)])
+def test_offline_checksum_passes(dt, logN, bs):
+    # the baseline of cufft_ft.h:19-95 (separate checksum passes around the transform): both passes
+    # against the same sums taken in fp64 by torch, agreement on a clean transform, and the shift a
+    # corrupted output element causes in its transform only
+    import torch
+    N = 1 << logN
+    rdt = torch.float32 if dt == "float2" else torch.float64
+    x = torch.view_as_complex(torch.rand((bs, N, 2), generator=torch.Generator(device="cuda").manual_seed(7 + logN),
+                                         device="cuda", dtype=rdt) * 2 - 1)
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    y = plan.fft(x).clone()
+    plan.close()
+    a, b = turbofft_amd.offline_checksums(x, y)
+    c = torch.from_numpy(turbofft_amd.checksum_vector(N, dt, "exact")).cuda().to(torch.complex128)
+    s3 = 0.8660253882408142
+    r = torch.tensor([1.0, -0.5 - 1j * s3, -0.5 + 1j * s3], dtype=torch.complex128, device="cuda")[torch.arange(N, device="cuda") % 3]
+    def re_plus_im(z):
+        return z.real + z.imag
+    a_ref = re_plus_im((x.to(torch.complex128) * c).sum(1))
+    b_ref = re_plus_im((y.to(torch.complex128) * r).sum(1))
+    eps = 1e-5 if dt == "float2" else 1e-13
+    scale = (x.abs().to(torch.float64) * c.abs()).sum(1) + (y.abs().to(torch.float64)).sum(1)
+    assert ((a.double() - a_ref).abs() <= eps * scale).all()
+    assert ((b.double() - b_ref).abs() <= eps * scale).all()
+    assert ((a.double() - b.double()).abs() <= 4 * eps * logN * scale).all()          # two-sided identity on clean data
+    row, k, e = bs // 2, (5 * N) // 7, 3.0
+    y[row, k] += e
+    a2, b2 = turbofft_amd.offline_checksums(x, y)
+    shift = (b2 - b).double()
+    want = torch.zeros(bs, dtype=torch.float64, device="cuda")
+    want[row] = re_plus_im(e * r[k]).item()
+    assert ((shift - want).abs() <= eps * scale + 1e-6).all()
+    # (transforms longer than 8192 points are summed from several partial sums in arrival order)
+    assert ((a2 - a).double().abs() <= eps * scale).all()
+
+
+def test_offline_ft_timing_runs_clean():
+    import torch
+    for dt, logN, bs in (("float2", 12, 256), ("double2", 17, 8)):
+        N = 1 << logN
+        x = torch.view_as_complex(torch.rand((bs, N, 2), device="cuda", dtype=torch.float32 if dt == "float2" else torch.float64) * 2 - 1)
+        out = torch.empty(2 * bs * N, dtype=x.dtype, device="cuda")
+        ms, flagged = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 1, 3,
+                                                   torch.cuda.current_stream().cuda_stream)
+        assert ms > 0 and flagged == 0
+        ref = torch.fft.fft(x.to(torch.complex128), dim=1)
+        got = out[: bs * N].view(bs, N).to(torch.complex128)
+        assert (torch.linalg.vector_norm(got - ref) / torch.linalg.vector_norm(ref)).item() < (1e-5 if dt == "float2" else 1e-13) * logN

@@ -140,6 +140,10 @@ def test_vendor_side_by_side_rejects_bad_arguments_before_touching_a_device():
     assert L.turbofft_vendor_time(10, 0, None, None, 4, 1, 10, None, ctypes.byref(ms)) != 0
     assert b"bad argument" in L.turbofft_last_error()
     assert turbofft_amd.vendor_available() in (True, False)      # opening the library needs no device
+    assert L.turbofft_offline_checksums(10, 0, None, None, 4, None, None, None) != 0
+    assert b"bad argument" in L.turbofft_last_error()
+    assert L.turbofft_offline_ft_time(10, 0, None, None, 4, 1, 10, None, ctypes.byref(ms), None) != 0
+    assert b"bad argument" in L.turbofft_last_error()
 
 
 def test_cli_help_and_bad_flag():

@@ -80,6 +80,8 @@ def lib() -> C.CDLL:
     L.turbofft_main.argtypes = [i, C.POINTER(C.c_char_p)]
     L.turbofft_vendor_exec.argtypes = [i, i, vp, vp, ll, vp]
     L.turbofft_vendor_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_offline_checksums.argtypes = [i, i, vp, vp, ll, vp, vp, vp]
+    L.turbofft_offline_ft_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_ulonglong)]
     _lib = L
     return L
 
@@ -141,6 +143,35 @@ def vendor_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, warmup:
     ms = C.c_float(0)
     _check(lib().turbofft_vendor_time(logN, _datatype(datatype), in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
     return ms.value
+
+
+# ---- offline checksums (the baseline of cufft/cufft_ft.h: separate passes around the transform) ----
+def offline_checksums(x, y):
+    """Per-transform input and output checksums of x -> y (both (bs, N) complex tensors on the
+    GPU), computed by two separate passes; returns two real tensors of length bs."""
+    import torch
+    if x.shape != y.shape or x.dim() != 2 or x.dtype != y.dtype or not (x.is_cuda and y.is_cuda) or \
+            not (x.is_contiguous() and y.is_contiguous()) or x.dtype not in (torch.complex64, torch.complex128):
+        raise ValueError("expected two contiguous complex tensors of the same (bs, N) shape on the GPU")
+    bs, N = x.shape
+    logN = N.bit_length() - 1
+    if N != 1 << logN:
+        raise ValueError("N must be a power of two")
+    rdt = torch.float32 if x.dtype == torch.complex64 else torch.float64
+    a = torch.empty(bs, dtype=rdt, device=x.device)
+    b = torch.empty(bs, dtype=rdt, device=x.device)
+    _check(lib().turbofft_offline_checksums(logN, FP32 if rdt == torch.float32 else FP64, x.data_ptr(), y.data_ptr(), bs,
+                                            a.data_ptr(), b.data_ptr(), torch.cuda.current_stream(x.device).cuda_stream))
+    return a, b
+
+
+def offline_ft_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0):
+    """(ms per execution, transforms flagged in the last one) of checksum pass + plain plan + checksum pass + compare."""
+    ms = C.c_float(0)
+    flagged = C.c_ulonglong(0)
+    _check(lib().turbofft_offline_ft_time(logN, _datatype(datatype), in_ptr, out_ptr, bs, warmup, reps, stream,
+                                          C.byref(ms), C.byref(flagged)))
+    return ms.value, flagged.value
 
 
 def turbofft_main(argv: List[str]) -> int:
