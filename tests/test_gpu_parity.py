@@ -251,6 +251,48 @@ def test_agrees_with_the_vendor_library(dt, logN, bs):
     plan.close()
 
 
+@pytest.mark.parametrize("dt,logN", [("float2", 26), ("float2", 29), ("double2", 27), ("double2", 29)])
+def test_plans_beyond_2p25(dt, logN):
+    # rows 26-29 (the reference's fp64 table lists them, param/A100/param_double2.csv:27-30; its
+    # dispatch stops at 2^25): one transform, checked with closed forms that need no second
+    # transform of that size -- a unit impulse at m gives W_N^(m k), the constant gives N at k = 0 --
+    # plus linearity on random data against the vendor library where that is available.
+    torch = _torch()
+    N = 1 << logN
+    rdt = torch.float32 if dt == "float2" else torch.float64
+    cdt = torch.complex64 if dt == "float2" else torch.complex128
+    eps = (1e-5 if dt == "float2" else 1e-13) * logN
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    assert plan.launches == 3
+    out = torch.empty(plan.out_elems(1), dtype=cdt, device="cuda")
+    x = torch.zeros((1, N), dtype=cdt, device="cuda")
+    m = (N // 3) | 1
+    x[0, m] = 1.0
+    y = plan.fft(x, out)
+    k = torch.arange(N, device="cuda", dtype=torch.int64)
+    ang = ((k * m) % N).to(torch.float64) * (-2.0 * np.pi / N)
+    err = max((y[0].real.double() - torch.cos(ang)).abs().max().item(), (y[0].imag.double() - torch.sin(ang)).abs().max().item())
+    print(f"{dt} 2^{logN}: impulse max abs error {err:.3e}", flush=True)
+    assert err <= eps
+    del ang, k
+    x.fill_(1.0)
+    y = plan.fft(x, out)
+    assert abs(y[0, 0].real.item() - N) <= eps * N and abs(y[0, 0].imag.item()) <= eps * N
+    y[0, 0] = 0
+    assert y.abs().max().item() <= eps * N
+    if turbofft_amd.vendor_available():
+        del x
+        x = torch.view_as_complex(torch.rand((1, N, 2), generator=torch.Generator(device="cuda").manual_seed(logN),
+                                             device="cuda", dtype=rdt) * 2 - 1)
+        ours = plan.fft(x, out)
+        theirs = turbofft_amd.vendor_fft(x)
+        theirs -= ours
+        err = (torch.linalg.vector_norm(theirs) / torch.linalg.vector_norm(ours)).item()
+        print(f"{dt} 2^{logN}: rel L2 difference to hipFFT {err:.3e}", flush=True)
+        assert err <= 2 * eps
+    plan.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT

@@ -44,8 +44,8 @@ def test_registry_has_every_kernel_of_the_builtin_plans():
 @pytest.mark.parametrize("dtype", ["float2", "double2"])
 def test_builtin_rows_match_csv_and_are_consistent(dtype):
     rows = P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}.csv"))
-    assert len(rows) >= 26
-    for logN in range(1, 26):
+    assert len(rows) == 30                               # the reference's tables end at 2^25 (fp32) / 2^29 (fp64)
+    for logN in range(1, 30):
         r = turbofft_amd.builtin_plan_row(dtype, logN)
         p = P.PlanRow.from_list(r)                       # the 11 reference columns
         full = rows[logN]                                # ... plus this build's optional flags
