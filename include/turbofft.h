@@ -72,6 +72,18 @@ void turbofft_plan_destroy(turbofft_plan_t* plan);
  * Stands in for the launch loop of test_turbofft (main.cu:46-49, 55-58). */
 int turbofft_exec(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs, void* stream);
 
+/* The unnormalised inverse transform, out[n] = sum_k in[k] exp(+2 pi i n k / N),
+ * with the same plan, buffers and rules as turbofft_exec (turbofft_exec_inverse
+ * of a turbofft_exec result is N times the input).  No counterpart in the
+ * reference, which is forward only (the sign is fixed in its twiddle table,
+ * initializeData.h:31-37, and in the generated butterflies).  inverse =
+ * swap(re,im) . forward . swap(re,im): the first launch runs a flavour of its
+ * kernel that exchanges re and im of what it loads, the last launch one that
+ * exchanges them before storing (compile-time flavours, built for the built-in
+ * plan rows).  Plain plans only: a fault-tolerant plan, or a caller's CSV whose
+ * inverse flavours were not built, returns TURBOFFT_ENOPLAN. */
+int turbofft_exec_inverse(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs, void* stream);
+
 /* Same, from and to host memory (allocates device buffers, copies, runs,
  * synchronises, frees).  Stands in for initializeData's H2D copy plus the
  * D2H copy at main.cu:72. */

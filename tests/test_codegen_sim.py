@@ -203,3 +203,19 @@ def test_cross_lane_last_pass(dtype, logNi, BS, n):
     ref = O.fft_ref(x.astype(simlib.ctype_of(dtype)))
     for b in range(bs):
         assert O.rel_l2(y[b], ref[b]) < O.tolerance(dtype, logNi)
+
+
+@pytest.mark.parametrize("dtype,logNi,BS,n,xl", [("float2", 10, 1, 16, 0), ("double2", 7, 4, 8, 0), ("double2", 11, 1, 8, 1)])
+def test_inverse_flavour_of_a_single_launch_kernel(dtype, logNi, BS, n, xl):
+    # the `_i` flavour exchanges re and im after the load and before the store, which turns the
+    # forward kernel into the unnormalised inverse transform
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 0, 0, 0, xl, 0, 0, 1))
+    assert sp.name.endswith("_i")
+    N = 1 << logNi
+    bs = BS * 3 + BS // 2
+    x = rnd((bs, N), logNi + 300)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = (bs + BS - 1) // BS, bs, 1, 1
+    y = simlib.run_sim(sp, x, bs * N, ka, ka.ntiles, simlib.twiddle_table(N, dtype)).reshape(bs, N)
+    ref = np.fft.ifft(x.astype(simlib.ctype_of(dtype)).astype(np.complex128), axis=1) * N
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)

@@ -293,6 +293,43 @@ def test_plans_beyond_2p25(dt, logN):
     plan.close()
 
 
+@pytest.mark.parametrize("dt,logN,bs", [("float2", 5, 1000), ("double2", 10, 16), ("double2", 11, 7), ("float2", 13, 33),
+                                        ("double2", 14, 4), ("float2", 17, 8), ("double2", 20, 2), ("float2", 24, 1)])
+def test_inverse_transform(dt, logN, bs):
+    # turbofft_exec_inverse: the unnormalised inverse (N * numpy's ifft) through component-swapping
+    # flavours of the forward kernels; one-, two- and three-launch plans (2^11 fp64 is the
+    # cross-lane kernel), then the round trip forward -> inverse = N * x
+    torch = _torch()
+    N = 1 << logN
+    rng = np.random.default_rng(400 + logN)
+    x = (rng.uniform(-1, 1, (bs, N)) + 1j * rng.uniform(-1, 1, (bs, N))).astype(cdtype(dt))
+    xd = torch.from_numpy(x).cuda()
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    y = plan.ifft(xd).cpu().numpy()
+    ref = np.fft.ifft(x.astype(np.complex128), axis=1) * N
+    err = O.rel_l2(y, ref)
+    print(f"{dt} logN={logN} bs={bs} launches={plan.launches}: inverse rel L2 {err:.3e}", flush=True)
+    assert err <= O.tolerance(dt, logN)
+    back = plan.ifft(plan.fft(xd).clone()).cpu().numpy() / N
+    assert O.rel_l2(back, x.astype(np.complex128)) <= 2 * O.tolerance(dt, logN)
+    plan.close()
+
+
+def test_inverse_transform_is_refused_where_it_was_not_built():
+    torch = _torch()
+    x = torch.zeros((4, 1024), dtype=torch.complex128, device="cuda")
+    plan = turbofft_amd.TurboFFT(10, "double2", if_ft=1, thread_bs=2)
+    with pytest.raises(turbofft_amd.TurboFFTError, match="inverse"):
+        plan.ifft(x)
+    plan.close()
+    shapes = os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param", "gfx950", "reference_shapes_double2.csv")
+    plan = turbofft_amd.TurboFFT(10, "double2", param_csv=shapes)          # n = 8: forward kernel only
+    with pytest.raises(turbofft_amd.TurboFFTError, match="inverse"):
+        plan.ifft(x)
+    plan.fft(x)
+    plan.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT

@@ -37,7 +37,7 @@ def test_registry_has_every_kernel_of_the_builtin_plans():
         for r in P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}_ft.csv")):
             assert rows[r.logN].launches > 0
             ft_rows[r.logN] = r
-        for key in collect_keys(rows, dtype, [0]) + collect_keys(ft_rows, dtype, [1]):
+        for key in collect_keys(rows, dtype, [0], inverse=True) + collect_keys(ft_rows, dtype, [1]):
             assert key.name in have
 
 
@@ -81,6 +81,15 @@ def test_optional_plan_columns():
     assert "GLDG(" in src and "GSTGN(" in src and "GLDGN(" not in src and "GSTG(" not in src
     with pytest.raises(ValueError):
         P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0] + [0] * 13 + [4])
+    # inverse plans: component-swapping flavours of the first and the last launch, plain only
+    r3 = P.PlanRow.from_list([24, 3, 8, 8, 8, 32, 16, 32, 32, 32, 32])
+    assert [k.name for k in P.kernels_for_row(r3, "float2", 0, inverse=True)] == \
+        ["tfft_f32_col_N8_b32_n32_i", "tfft_f32_col_N8_b16_n32", "tfft_f32_rowT_N8_b32_n32_i"]
+    with pytest.raises(ValueError):
+        P.kernels_for_row(r3, "float2", 1, inverse=True)
+    fwd = generate_source([KernelSpec(P.kernels_for_row(r3, "float2", 0)[0])], False)
+    inv = generate_source([KernelSpec(P.kernels_for_row(r3, "float2", 0, inverse=True)[0])], False)
+    assert "cswap(" not in fwd and inv.count("cswap(") == 32
     short = P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0])
     assert (short.split, short.tiles, short.wv) == ((0,), 0, (0,))
     assert "amdgpu_waves_per_eu" not in generate_source([KernelSpec(P.kernels_for_row(short, "float2", 0)[0])], False)

@@ -59,6 +59,7 @@ def lib() -> C.CDLL:
     L.turbofft_plan_destroy.argtypes = [vp]
     L.turbofft_plan_destroy.restype = None
     L.turbofft_exec.argtypes = [vp, vp, vp, ll, vp]
+    L.turbofft_exec_inverse.argtypes = [vp, vp, vp, ll, vp]
     L.turbofft_exec_host.argtypes = [vp, vp, vp, ll]
     L.turbofft_time.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_time_launches.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
@@ -237,7 +238,14 @@ class TurboFFT:
     def exec(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
         _check(lib().turbofft_exec(self._h, in_ptr, out_ptr, bs, stream))
 
-    def fft(self, x, out=None):
+    def exec_inverse(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
+        _check(lib().turbofft_exec_inverse(self._h, in_ptr, out_ptr, bs, stream))
+
+    def ifft(self, x, out=None):
+        """Unnormalised inverse transform (N times numpy's ifft); arguments as for fft()."""
+        return self.fft(x, out, _inverse=True)
+
+    def fft(self, x, out=None, _inverse=False):
         """x: torch tensor on the GPU, shape (bs, N), complex64/complex128.
         Returns a (bs, N) view of the transform (natural order)."""
         import torch
@@ -251,7 +259,7 @@ class TurboFFT:
             out = torch.empty(self.out_elems(bs), dtype=want, device=x.device)
         elif out.numel() < self.out_elems(bs) or out.dtype != want or not out.is_contiguous():
             raise ValueError(f"out must be contiguous {want} with >= {self.out_elems(bs)} elements")
-        self.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream(x.device).cuda_stream)
+        (self.exec_inverse if _inverse else self.exec)(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream(x.device).cuda_stream)
         return out.view(-1)[: bs * self.N].view(bs, self.N)
 
     def fft_host(self, x: np.ndarray) -> np.ndarray:

@@ -74,12 +74,15 @@ class KernelKey:
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
     wv: int = 0      # > 0: compiled to fit this many wavefronts per SIMD (register budget 512 / wv)
     nt: int = 0      # bit 0: tile loads are non-temporal, bit 1: tile stores are
+    inv: int = 0     # 1: the flavour an inverse plan uses in this position -- re and im exchanged as
+                     # they are loaded (row1, col as first launch) and/or before they are stored
+                     # (row1, rowT): inverse = swap . forward . swap
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_ft" if self.ft else ""))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ("_ft" if self.ft else ""))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:
@@ -97,7 +100,12 @@ def launch_kinds(launches: int) -> List[str]:
     return {1: ["row1"], 2: ["col", "rowT"], 3: ["col", "col", "rowT"]}[launches]
 
 
-def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
+def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False) -> List[KernelKey]:
+    """Kernels of the row's launches; with `inverse` the first and the last launch use their
+    component-swapping flavour (plain plans only), launches in between are the forward ones."""
+    if inverse and ft:
+        raise ValueError("inverse plans have no fault-tolerant flavour")
+    last = row.launches - 1
     return [KernelKey(dtype, kind, row.logNi[i], row.BS[i], row.n[i], int(ft), int(row.split[i]) if row.split else 0,
                       int(row.pf[i]) if row.pf else 0,
                       # fault-tolerant plans keep the LDS path: the checksum model fixes which
@@ -106,7 +114,8 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int) -> List[KernelKey]:
                       # the register budget hint was tuned on the plain kernel only (fault-tolerant
                       # kernels keep their table in registers and spill under any tighter budget)
                       (int(row.wv[i]) if row.wv else 0) if not ft else 0,
-                      int(row.nt[i]) if row.nt else 0)
+                      int(row.nt[i]) if row.nt else 0,
+                      1 if inverse and i in (0, last) else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 
 

@@ -130,6 +130,7 @@ TFFT_DEV float2 cmul_mi(float2 a) { float2 c; c.x = a.y; c.y = -a.x; return c; }
 TFFT_DEV float2 cmul_pi(float2 a) { float2 c; c.x = -a.y; c.y = a.x; return c; }   // * (+i)
 TFFT_DEV float2 cneg(float2 a) { float2 c; c.x = -a.x; c.y = -a.y; return c; }
 TFFT_DEV float2 czero(float2) { float2 c; c.x = 0.f; c.y = 0.f; return c; }
+TFFT_DEV float2 cswap(float2 a) { float2 c; c.x = a.y; c.y = a.x; return c; }       // (re, im) -> (im, re)
 
 TFFT_DEV double2 cadd(double2 a, double2 b) { double2 c; c.x = a.x + b.x; c.y = a.y + b.y; return c; }
 TFFT_DEV double2 csub(double2 a, double2 b) { double2 c; c.x = a.x - b.x; c.y = a.y - b.y; return c; }
@@ -139,6 +140,7 @@ TFFT_DEV double2 cmul_mi(double2 a) { double2 c; c.x = a.y; c.y = -a.x; return c
 TFFT_DEV double2 cmul_pi(double2 a) { double2 c; c.x = -a.y; c.y = a.x; return c; }
 TFFT_DEV double2 cneg(double2 a) { double2 c; c.x = -a.x; c.y = -a.y; return c; }
 TFFT_DEV double2 czero(double2) { double2 c; c.x = 0.0; c.y = 0.0; return c; }
+TFFT_DEV double2 cswap(double2 a) { double2 c; c.x = a.y; c.y = a.x; return c; }
 
 #ifndef TFFT_SIM
 // Cross-lane fetch of the value held by lane (lane ^ MASK): DPP quad permutes for

@@ -102,12 +102,12 @@ int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
     return i == launches - 1 ? 2 : 1;
 }
 
-const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv, int nt) {
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv, int nt, int inv = 0) {
     int cnt = 0;
     const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
-            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt)
+            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt && t[i].inv == inv)
             return &t[i];
     return nullptr;
 }
@@ -187,6 +187,7 @@ struct turbofft_plan {
     Row row{};
     int launches = 0;
     const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
+    const tfft_kernel_entry* k_inv[3] = {nullptr, nullptr, nullptr};   // inverse plans: flavour of launch i (first and last differ from k)
     int tb_gap[3] = {1, 1, 1};
     int resident[3] = {1, 1, 1};   // blocks of launch i that fit on the device at once
     size_t esize = 8;
@@ -327,6 +328,18 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
         p->k[i] = k;
+        // Inverse plans run the same launches with a component-swapping flavour of the first and
+        // the last one (plain plans only; absent for a caller's CSV whose kernels were built
+        // without them, and then turbofft_exec_inverse reports it).
+        p->k_inv[i] = k;
+        if (!p->if_ft && (i == 0 || i == p->launches - 1)) {
+            p->k_inv[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 0, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
+                                      r.xl(i) ? 1 : 0, r.wv(i), r.nt(i), 1);
+            if (p->k_inv[i] && (size_t)p->k_inv[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
+                HIP_TRY(hipFuncSetAttribute(p->k_inv[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_inv[i]->lds_bytes));
+        } else if (p->if_ft) {
+            p->k_inv[i] = nullptr;
+        }
         if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
             HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
         int nb = 0;
@@ -521,15 +534,27 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
     return TURBOFFT_OK;
 }
 
-static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev);
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev,
+                     bool inverse = false);
 
 int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
     return exec_impl(p, in_d, out_d, bs, stream, nullptr);
 }
 
+int turbofft_exec_inverse(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
+    return exec_impl(p, in_d, out_d, bs, stream, nullptr, true);
+}
+
 // ev (optional): launches+1 events; ev[i] is recorded before launch i, ev[launches] after the last
-static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev) {
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev,
+                     bool inverse) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (inverse) {
+        if (p->if_ft) return fail(TURBOFFT_ENOPLAN, "fault-tolerant plans have no inverse kernels");
+        for (int i = 0; i < p->launches; ++i)
+            if (!p->k_inv[i])
+                return fail(TURBOFFT_ENOPLAN, "no compiled inverse kernel for launch %d of logN=%d (built for the built-in plan rows only)", i, p->logN);
+    }
     if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
     if (bs == 0) return TURBOFFT_OK;
     if (!in_d || !out_d) return fail(TURBOFFT_EINVAL, "null buffer");
@@ -545,7 +570,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     else if (p->launches == 2) { src[0] = in_d; dst[0] = work; src[1] = work; dst[1] = out; }
     else { src[0] = in_d; dst[0] = out; src[1] = out; dst[1] = work; src[2] = work; dst[2] = out; }
     for (int i = 0; i < p->launches; ++i) {
-        const tfft_kernel_entry* k = p->k[i];
+        const tfft_kernel_entry* k = inverse ? p->k_inv[i] : p->k[i];
         tfft_kargs a;
         memset(&a, 0, sizeof a);
         a.ntiles = launch_tiles(p, i, bs);
