@@ -8,7 +8,6 @@
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
-#include <cstdio>
 #include <mutex>
 
 #include "../../include/turbofft.h"
@@ -19,12 +18,10 @@ namespace {
 
 // the part of the hipFFT C API that is used (hipfft/hipfft.h); handles are opaque pointers
 typedef void* vfft_handle;
-typedef int (*fn_create)(vfft_handle*);
 typedef int (*fn_plan1d)(vfft_handle*, int, int, int);
 typedef int (*fn_set_stream)(vfft_handle, hipStream_t);
 typedef int (*fn_exec)(vfft_handle, void*, void*, int);
 typedef int (*fn_destroy)(vfft_handle);
-typedef int (*fn_version)(int*);
 constexpr int VFFT_C2C = 0x29, VFFT_Z2Z = 0x69, VFFT_FORWARD = -1;
 
 struct VendorLib {
@@ -33,7 +30,6 @@ struct VendorLib {
     fn_set_stream set_stream = nullptr;
     fn_exec exec_c2c = nullptr, exec_z2z = nullptr;
     fn_destroy destroy = nullptr;
-    fn_version version = nullptr;
     bool tried = false;
 };
 VendorLib g_lib;
@@ -53,7 +49,6 @@ bool load_vendor() {
     g_lib.exec_c2c = (fn_exec)dlsym(so, "hipfftExecC2C");
     g_lib.exec_z2z = (fn_exec)dlsym(so, "hipfftExecZ2Z");
     g_lib.destroy = (fn_destroy)dlsym(so, "hipfftDestroy");
-    g_lib.version = (fn_version)dlsym(so, "hipfftGetVersion");
     if (!g_lib.plan1d || !g_lib.set_stream || !g_lib.exec_c2c || !g_lib.exec_z2z || !g_lib.destroy) {
         dlclose(so);
         return false;
@@ -120,14 +115,15 @@ extern "C" int turbofft_vendor_time(int logN, int datatype, const void* in_d, vo
         tfft_set_error("vendor FFT: event creation failed");
         return TURBOFFT_EHIP;
     }
-    rc = hipEventRecord(e0, st) == hipSuccess ? 0 : TURBOFFT_EHIP;
-    for (int i = 0; i < reps && !rc; ++i) rc = run(p, datatype, in_d, out_d);
-    if (!rc && (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess)) rc = TURBOFFT_EHIP;
     float ms = 0;
-    if (!rc && hipEventElapsedTime(&ms, e0, e1) != hipSuccess) rc = TURBOFFT_EHIP;
+    bool timed = hipEventRecord(e0, st) == hipSuccess;
+    for (int i = 0; i < reps && timed && !rc; ++i) rc = run(p, datatype, in_d, out_d);     // run() sets the message
+    timed = timed && !rc && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+            hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    if (rc == TURBOFFT_EHIP && hipGetLastError() != hipSuccess) tfft_set_error("vendor FFT: timing failed");
-    if (!rc) *ms_per_exec = ms / (float)reps;
-    return rc;
+    if (rc) return rc;
+    if (!timed) { tfft_set_error("vendor FFT: event timing failed"); return TURBOFFT_EHIP; }
+    *ms_per_exec = ms / (float)reps;
+    return 0;
 }
