@@ -55,11 +55,12 @@ const char* turbofft_last_error(void);
  *              fault tolerance it only shapes the grid; 1 (the reference's
  *              default) then lets the plan row use its own tuned value.
  *   param_csv  plan CSV in the reference's 11-column format, row index ==
- *              logN; NULL selects the built-in gfx950 table.  Up to 16 more
+ *              logN; NULL selects the built-in gfx950 table.  Up to 19 more
  *              columns per row are optional tuning flags of this library
  *              (per-launch split exchange, prefetch, cross-lane last pass,
  *              tiles per block, per-launch wavefronts per SIMD, per-launch
- *              non-temporal accesses); a reference CSV without them is valid.
+ *              non-temporal accesses, per-launch tiles per XCD); a reference
+ *              CSV without them is valid.
  * Returns NULL on error. */
 turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_err,
                                       int thread_bs, const char* param_csv);

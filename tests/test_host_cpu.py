@@ -81,6 +81,10 @@ def test_optional_plan_columns():
     assert "GLDG(" in src and "GSTGN(" in src and "GLDGN(" not in src and "GSTG(" not in src
     with pytest.raises(ValueError):
         P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0] + [0] * 13 + [4])
+    # columns 28-30: tiles per XCD, a launch parameter (no kernel depends on it)
+    r = P.PlanRow.from_list([20, 2, 10, 10, 0, 16, 16, 0, 32, 32, 0] + [0] * 16 + [8, 32])
+    assert r.xc == (8, 32)
+    assert [k.name for k in P.kernels_for_row(r, "float2", 0)] == ["tfft_f32_col_N10_b16_n32", "tfft_f32_rowT_N10_b16_n32"]
     # inverse plans: component-swapping flavours of the first and the last launch, plain only
     r3 = P.PlanRow.from_list([24, 3, 8, 8, 8, 32, 16, 32, 32, 32, 32])
     assert [k.name for k in P.kernels_for_row(r3, "float2", 0, inverse=True)] == \

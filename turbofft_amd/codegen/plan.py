@@ -12,7 +12,9 @@ walks when the caller leaves thread_bs at 1 (0 or absent: one); columns 22-24
 `w1, w2, w3` ask the compiler to fit that many wavefronts per SIMD (0: its own
 choice) for the plain kernel of the launch; columns 25-27 `t1, t2, t3` mark the
 launch's tile loads (1), stores (2) or both (3) as non-temporal (streamed past the
-caches; tables and twiddles stay cached).  Launch i transforms a digit of size 2^logNi with BSi
+caches; tables and twiddles stay cached); columns 28-30 `g1, g2, g3` give the number of
+consecutive tiles each of the 8 XCDs works on in that launch (a run-time launch parameter,
+0 = 64).  Launch i transforms a digit of size 2^logNi with BSi
 sub-FFTs per tile and ni elements per thread; launch 0 owns the most-strided
 digit and the last launch the contiguous one.
 """
@@ -35,6 +37,7 @@ class PlanRow:
     tiles: int = 0                   # optional column 21: tiles per block of the plain plan (0 = 1)
     wv: Tuple[int, ...] = ()         # optional columns 22-24: wavefronts per SIMD to compile for (0 = free)
     nt: Tuple[int, ...] = ()         # optional columns 25-27: 1 = non-temporal tile loads, 2 = stores, 3 = both
+    xc: Tuple[int, ...] = ()         # optional columns 28-30: consecutive tiles per XCD (run time only; 0 = 64)
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -49,7 +52,7 @@ class PlanRow:
         ext3 = (row[17:20] + [0, 0, 0])[:3]
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
                     tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
-                    tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]))
+                    tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]), tuple((row[27:30] + [0, 0, 0])[:L]))
         if any(t not in (0, 1, 2, 3) for t in p.nt):
             raise ValueError(f"non-temporal columns must be 0..3 in row {row}")
         if L and sum(p.logNi) != p.logN:
@@ -92,7 +95,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:27] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:30] if t.strip()]))
     return rows
 
 

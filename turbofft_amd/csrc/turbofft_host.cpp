@@ -62,11 +62,13 @@ constexpr double kPi = 3.14159265358979323846;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[27];           // 11 reference columns + optional per-launch flags: split exchange,
+    int v[30];           // 11 reference columns + optional per-launch flags: split exchange,
                          // prefetch, cross-lane last pass; then the tiles-per-block hint, the
                          // per-launch wavefronts-per-SIMD the plain kernel was compiled for and
-                         // the per-launch non-temporal access bits
+                         // the per-launch non-temporal access bits, then the per-launch
+                         // number of consecutive tiles an XCD works on (0 = 64)
     int nt(int i) const { return v[24 + i]; }
+    int xc(int i) const { return v[27 + i]; }
     int tiles() const { return v[20]; }
     int wv(int i) const { return v[21 + i]; }
     int split(int i) const { return v[11 + i]; }
@@ -90,7 +92,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 27 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 30 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -207,7 +209,8 @@ struct turbofft_plan {
     long long inj_tile = 0;
     double inj_mag = 100.0;
     int cksum_mode = 0;
-    int xcd_chunk = 64;          // tiles per XCD chunk (0 = plain block order)
+    int xcd_chunk = -1;          // TURBOFFT_XCD_CHUNK: tiles per XCD chunk for every launch (0 = plain block order); -1 = unset
+    int xcd_chunk_l[3] = {64, 64, 64};   // per launch: the plan row's value, else 64
     unsigned long long checked = 0;   // checksum groups launched since the last reset
 };
 
@@ -328,6 +331,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
         p->k[i] = k;
+        if (r.xc(i) > 0) p->xcd_chunk_l[i] = r.xc(i);
         // Inverse plans run the same launches with a component-swapping flavour of the first and
         // the last one (plain plans only; absent for a caller's CSV whose kernels were built
         // without them, and then turbofft_exec_inverse reports it).
@@ -583,7 +587,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.tb_gap = p->resident[i];
             a.thread_bs = (int)((a.ntiles + p->resident[i] - 1) / p->resident[i]);
         }
-        a.xcd_chunk = p->xcd_chunk;
+        a.xcd_chunk = p->xcd_chunk >= 0 ? p->xcd_chunk : p->xcd_chunk_l[i];
         int kind = kind_of_launch(p->launches, i);
         if (kind == 1) {
             int log_ncols = 0;
