@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the batched FFT hot path on one MI355X.
 
-Default workload: BASELINE config 2 -- forward C2C FFT, fp32 complex, N=2^13,
+Default workload: benchmark configuration 2 -- forward C2C FFT, fp32 complex, N=2^13,
 batch 2^15 (logBS+logN=28, 2 GiB in, 2 GiB out), synthetic uniform[-1,1) data
 resident in HBM before the timed region.  A "step" is one transform of the
 whole batch.  Prints ONE JSON line:

@@ -177,7 +177,7 @@ def _model_groups_last_launch(xsel, row, dt, groups, tiles_per_transform, injs, 
 
 
 def test_config5_fp64_2p20_batch256():
-    # BASELINE config 5: fp64, N=2^20, batch 256, threshold 1e-3, err_smoothing 1000, one
+    # benchmark configuration 5: fp64, N=2^20, batch 256, threshold 1e-3, err_smoothing 1000, one
     # error in 1 of every 1000 tile groups of the last launch.  Run (i) with the stated
     # magnitude 100 and (ii) with an error sized above the rule's floor for this data;
     # the decisions of every group that holds an injected tile must equal the oracle model's.

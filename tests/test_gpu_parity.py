@@ -45,7 +45,7 @@ SHAPES_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file
 
 
 def test_config1_fp64_2p10_batch16():
-    # BASELINE config 1: fp64, N=2^10, batch 16, U[-1,1) seed 0, single launch n=8 -- with the
+    # benchmark configuration 1: fp64, N=2^10, batch 16, U[-1,1) seed 0, single launch n=8 -- with the
     # plan shape the configuration names, and with the built-in row for this size
     x = make(16, 1024, "double2", 0)
     shaped = turbofft_amd.TurboFFT(10, "double2", param_csv=os.path.join(SHAPES_DIR, "reference_shapes_double2.csv"))
@@ -56,7 +56,7 @@ def test_config1_fp64_2p10_batch16():
 
 
 def test_config3_and_config4_plan_shapes():
-    # BASELINE config 3 (fp64 2^15, two launches 7/8 with BS 16/8, standard normal input) and
+    # benchmark configuration 3 (fp64 2^15, two launches 7/8 with BS 16/8, standard normal input) and
     # config 4 (fp32 2^24, three launches 8/8/8 with BS 16): the named plan shapes on a few
     # transforms; the full 2^28-point sizes of these plans are covered by the sweeps below
     rng = np.random.default_rng(3)
@@ -151,7 +151,7 @@ def test_input_is_not_modified():
 
 
 def test_config2_full_size_fp32_2p13():
-    # BASELINE config 2 at full size (2^28 points): sampled batches against the oracle,
+    # benchmark configuration 2 at full size (2^28 points): sampled batches against the oracle,
     # plus linearity of the whole batch as a size-independent property
     torch = _torch()
     logN, bs = 13, 1 << 15
@@ -204,14 +204,14 @@ def _full_size_check(torch, plan, dt, logN, bs, normal):
 
 
 def test_config3_full_size_fp64_2p15():
-    # BASELINE config 3 at full size: fp64, N=2^15, batch 2^13, standard normal input, two launches
+    # benchmark configuration 3 at full size: fp64, N=2^15, batch 2^13, standard normal input, two launches
     plan = turbofft_amd.TurboFFT(15, "double2")
     assert plan.launches == 2
     _full_size_check(_torch(), plan, "double2", 15, 1 << 13, normal=True)
 
 
 def test_config4_full_size_fp32_2p24():
-    # BASELINE config 4 at full size: fp32, N=2^24, batch 16, three launches
+    # benchmark configuration 4 at full size: fp32, N=2^24, batch 16, three launches
     plan = turbofft_amd.TurboFFT(24, "float2")
     assert plan.launches == 3
     _full_size_check(_torch(), plan, "float2", 24, 16, normal=False)

@@ -120,7 +120,7 @@ PLANS = [
     [6, 3, 2, 2, 2, 2, 2, 2, 2, 4, 4],          # 4 x 4 x 4
     [7, 2, 3, 4, 0, 4, 2, 0, 8, 4, 0],          # unequal digits: transposed operand fails
     [9, 3, 2, 3, 4, 4, 2, 2, 4, 8, 4],          # all digits different
-    [15, 2, 7, 8, 0, 16, 8, 0, 8, 8, 0],        # BASELINE config 3 row
+    [15, 2, 7, 8, 0, 16, 8, 0, 8, 8, 0],        # benchmark configuration 3 row
 ]
 
 
