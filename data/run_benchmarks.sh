@@ -10,10 +10,14 @@ out=${1:-data}
 bin=turbofft_amd/bin/turbofft
 gpu=MI355X
 mkdir -p "$out/ft"
-run() {   # run <file> <line prefix> <flags...>: keep the metric lines only, as the reference's files do
+run() {   # run <file> <line prefix> <flags...>: keep the metric lines only, as the reference's files do,
+          # as a CSV with a header and the fraction of the 8 TB/s HBM peak as a last column
     local file=$1 prefix=$2; shift 2
     echo "$file" >&2
-    timeout -k 10 300 "$bin" "$@" --gpu $gpu | grep "^$prefix" > "$file" || { echo "failed: $bin $*" >&2; exit 1; }
+    timeout -k 10 300 "$bin" "$@" --gpu $gpu | grep "^$prefix" |
+        awk -F', *' 'BEGIN { print "library,logN,log2_batch,ms,GFLOPS,GBps,pct_of_hbm_peak" }
+                     { printf "%s,%d,%d,%.3f,%.3f,%.3f,%.2f\n", $1, $2, $3, $4, $5, $6, $6 / 80.0 }' > "$file"
+    [ "$(wc -l < "$file")" -gt 1 ] || { echo "failed: $bin $*" >&2; exit 1; }
 }
 for dt in 0 1; do
     p=$([ $dt = 0 ] && echo fp32 || echo fp64)
