@@ -22,7 +22,9 @@ def rnd(shape, seed):
 
 ROW1 = [("double2", 10, 1, 8), ("float2", 10, 1, 16), ("float2", 13, 1, 32), ("double2", 7, 4, 8),
         ("float2", 7, 8, 8), ("float2", 3, 64, 4), ("double2", 1, 128, 2), ("float2", 4, 16, 4),
-        ("double2", 12, 1, 16), ("float2", 8, 4, 16), ("float2", 6, 32, 32)]
+        ("double2", 12, 1, 16), ("float2", 8, 4, 16), ("float2", 6, 32, 32),
+        # one whole transform per thread: fp32 kernels of this shape move two elements per access
+        ("float2", 1, 256, 2), ("float2", 2, 64, 4), ("float2", 3, 128, 8), ("float2", 4, 64, 16)]
 
 
 @pytest.mark.parametrize("dtype,logNi,BS,n", ROW1)

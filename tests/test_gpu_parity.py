@@ -330,6 +330,28 @@ def test_inverse_transform_is_refused_where_it_was_not_built():
     plan.close()
 
 
+def test_whole_transform_threads_need_aligned_buffers():
+    # fp32 plans whose threads hold whole transforms (2 and 4 points in the built-in table) move
+    # two elements per 128-bit access: a buffer that starts on an odd element is refused before
+    # anything is launched, an aligned one is transformed
+    torch = _torch()
+    for logN in (1, 2):
+        N = 1 << logN
+        xh = make(1000, N, "float2", logN)
+        x = torch.from_numpy(np.append(xh.reshape(-1), np.complex64(0))).cuda()
+        out = torch.empty(1000 * N + 1, dtype=torch.complex64, device="cuda")
+        plan = turbofft_amd.TurboFFT(logN, "float2")
+        st = torch.cuda.current_stream().cuda_stream
+        with pytest.raises(turbofft_amd.TurboFFTError, match="aligned"):
+            plan.exec(x.data_ptr() + 8, out.data_ptr(), 1000, st)
+        with pytest.raises(turbofft_amd.TurboFFTError, match="aligned"):
+            plan.exec(x.data_ptr(), out.data_ptr() + 8, 1000, st)
+        plan.exec(x.data_ptr(), out.data_ptr(), 1000, st)
+        torch.cuda.synchronize()
+        assert O.rel_l2(out[:1000 * N].cpu().numpy().reshape(1000, N), O.fft_ref(xh)) <= O.tolerance("float2", logN)
+        plan.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT

@@ -196,6 +196,13 @@ class KernelEmitter:
             self.GST += "N"
         self.TWL, self.TWLU = ("TWLD", "TWLDU") if buf else ("TWLG", "TWLGU")
 
+    def pair_access(self) -> bool:
+        """Whether a thread reads and writes its elements two at a time (one 128-bit access):
+        fp32 kernels whose threads hold whole transforms, where a lane's elements are
+        contiguous in memory.  fp64 elements already fill a 128-bit access."""
+        sp = self.s
+        return sp.kind == "row1" and sp.Tr == 1 and self.T2 == "float2" and sp.n % 2 == 0
+
     # ---------- literals ----------
     def lit(self, v: float) -> str:
         if self.R == "float":
@@ -418,8 +425,12 @@ class KernelEmitter:
             if sp.BS > 1:
                 c(f"if ((row0{sfx} + s) < a.nrows) {{")
                 c.ind += 1
-            for e in range(sp.n):
-                c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
+            if self.pair_access():
+                for e in range(0, sp.n, 2):
+                    c(f"{self.GLD}2(in, ubase{sfx}, {e}, gi{sfx}, {dst}[{e}], {dst}[{e + 1}]);")
+            else:
+                for e in range(sp.n):
+                    c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
             if sp.BS > 1:
                 c.ind -= 1
                 c("} else {")
@@ -468,8 +479,12 @@ class KernelEmitter:
             if sp.BS > 1:
                 c("if ((row0 + s) < a.nrows) {")
                 c.ind += 1
-            for e in range(sp.n):
-                c(f"{self.GST}(out, ubase, {sp.Tr * e}, go, r[{self.out_reg(e)}]);")
+            if self.pair_access():
+                for e in range(0, sp.n, 2):
+                    c(f"{self.GST}2(out, ubase, {e}, go, r[{self.out_reg(e)}], r[{self.out_reg(e + 1)}]);")
+            else:
+                for e in range(sp.n):
+                    c(f"{self.GST}(out, ubase, {sp.Tr * e}, go, r[{self.out_reg(e)}]);")
             if sp.BS > 1:
                 c.ind -= 1
                 c("}")

@@ -47,7 +47,24 @@ __device__ __forceinline__ void tfft_bst(double2* p, unsigned voff, unsigned sof
     t.z = (unsigned)__double2loint(v.y); t.w = (unsigned)__double2hiint(v.y);
     __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, AUX);
 }
+// Two adjacent fp32 elements in one 128-bit access: for kernels whose threads hold whole
+// transforms, so that a lane's elements are contiguous.  The byte address must be a multiple
+// of 16 (the host checks the tensor pointers of plans that use these).
+template <int AUX = 0>
+__device__ __forceinline__ void tfft_bld2(const float2* p, unsigned voff, unsigned soff, float2& a, float2& b) {
+    const tfft_u4 t = __builtin_amdgcn_raw_buffer_load_b128(tfft_rsrc(p), voff, soff, AUX);
+    a.x = __uint_as_float(t.x); a.y = __uint_as_float(t.y); b.x = __uint_as_float(t.z); b.y = __uint_as_float(t.w);
+}
+template <int AUX = 0>
+__device__ __forceinline__ void tfft_bst2(float2* p, unsigned voff, unsigned soff, float2 a, float2 b) {
+    tfft_u4 t; t.x = __float_as_uint(a.x); t.y = __float_as_uint(a.y); t.z = __float_as_uint(b.x); t.w = __float_as_uint(b.y);
+    __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, AUX);
+}
 #define TFFT_ESZ(p) ((unsigned)sizeof(*(p)))
+#define GLDU2(p, ub, uo, off, A, B) tfft_bld2<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
+#define GSTU2(p, ub, uo, off, A, B) tfft_bst2<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
+#define GLDUN2(p, ub, uo, off, A, B) tfft_bld2<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
+#define GSTUN2(p, ub, uo, off, A, B) tfft_bst2<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
 #define GLDU(p, ub, uo, off) tfft_bld<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
 #define GSTU(p, ub, uo, off, v) tfft_bst<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
 // the same accesses marked non-temporal: tile data is touched once, so it need not displace
@@ -108,6 +125,10 @@ extern long long tfft_sim_errors;
 #define GSTUN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
 #define GLDGN(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTGN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
+#define GLDU2(p, ub, uo, off, A, B) { (A) = GLDU(p, ub, uo, off); (B) = GLDU(p, ub, (uo) + 1, off); }
+#define GSTU2(p, ub, uo, off, A, B) { GSTU(p, ub, uo, off, A); GSTU(p, ub, (uo) + 1, off, B); }
+#define GLDUN2(p, ub, uo, off, A, B) GLDU2(p, ub, uo, off, A, B)
+#define GSTUN2(p, ub, uo, off, A, B) GSTU2(p, ub, uo, off, A, B)
 #define TWLG(p, i) TWLD(p, i)
 #define TWLGU(p, c, i) TWLDU(p, c, i)
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
