@@ -330,25 +330,30 @@ def test_inverse_transform_is_refused_where_it_was_not_built():
     plan.close()
 
 
-def test_whole_transform_threads_need_aligned_buffers():
+def test_whole_transform_threads_take_any_buffer_alignment():
     # fp32 plans whose threads hold whole transforms (2 and 4 points in the built-in table) move
-    # two elements per 128-bit access: a buffer that starts on an odd element is refused before
-    # anything is launched, an aligned one is transformed
+    # two elements per 128-bit access when a buffer is aligned to 16 bytes and one element per
+    # access otherwise: all four combinations of aligned and odd-element buffers give the same bits
     torch = _torch()
     for logN in (1, 2):
         N = 1 << logN
         xh = make(1000, N, "float2", logN)
-        x = torch.from_numpy(np.append(xh.reshape(-1), np.complex64(0))).cuda()
-        out = torch.empty(1000 * N + 1, dtype=torch.complex64, device="cuda")
+        x = torch.from_numpy(np.append(np.complex64(0), xh.reshape(-1))).cuda()   # data from element 1
+        xa = x[1:].clone()                                                      # the same data, aligned
         plan = turbofft_amd.TurboFFT(logN, "float2")
         st = torch.cuda.current_stream().cuda_stream
-        with pytest.raises(turbofft_amd.TurboFFTError, match="aligned"):
-            plan.exec(x.data_ptr() + 8, out.data_ptr(), 1000, st)
-        with pytest.raises(turbofft_amd.TurboFFTError, match="aligned"):
-            plan.exec(x.data_ptr(), out.data_ptr() + 8, 1000, st)
-        plan.exec(x.data_ptr(), out.data_ptr(), 1000, st)
-        torch.cuda.synchronize()
-        assert O.rel_l2(out[:1000 * N].cpu().numpy().reshape(1000, N), O.fft_ref(xh)) <= O.tolerance("float2", logN)
+        results = []
+        for src in (xa.data_ptr(), x.data_ptr() + 8):
+            for shift in (0, 1):
+                out = torch.zeros(1000 * N + 2, dtype=torch.complex64, device="cuda")
+                plan.exec(src, out.data_ptr() + 8 * shift, 1000, st)
+                torch.cuda.synchronize()
+                got = out.cpu().numpy()
+                assert got[:shift].tolist() == [0] * shift and got[shift + 1000 * N:].tolist() == [0] * (2 - shift)
+                results.append(got[shift:shift + 1000 * N].reshape(1000, N))
+        assert O.rel_l2(results[0], O.fft_ref(xh)) <= O.tolerance("float2", logN)
+        for r in results[1:]:
+            assert np.array_equal(r.view(np.uint32), results[0].view(np.uint32))
         plan.close()
 
 

@@ -197,9 +197,10 @@ class KernelEmitter:
         self.TWL, self.TWLU = ("TWLD", "TWLDU") if buf else ("TWLG", "TWLGU")
 
     def pair_access(self) -> bool:
-        """Whether a thread reads and writes its elements two at a time (one 128-bit access):
-        fp32 kernels whose threads hold whole transforms, where a lane's elements are
-        contiguous in memory.  fp64 elements already fill a 128-bit access."""
+        """Whether a thread reads and writes its elements two at a time (one 128-bit access)
+        when the buffer is aligned to 16 bytes: fp32 kernels whose threads hold whole
+        transforms, where a lane's elements are contiguous in memory.  fp64 elements already
+        fill a 128-bit access."""
         sp = self.s
         return sp.kind == "row1" and sp.Tr == 1 and self.T2 == "float2" and sp.n % 2 == 0
 
@@ -426,11 +427,19 @@ class KernelEmitter:
                 c(f"if ((row0{sfx} + s) < a.nrows) {{")
                 c.ind += 1
             if self.pair_access():
+                # a buffer that starts on an odd element takes the one-element accesses (uniform branch)
+                c("if (((unsigned long long)in & 15ull) == 0ull) {")
+                c.ind += 1
                 for e in range(0, sp.n, 2):
                     c(f"{self.GLD}2(in, ubase{sfx}, {e}, gi{sfx}, {dst}[{e}], {dst}[{e + 1}]);")
-            else:
-                for e in range(sp.n):
-                    c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
+                c.ind -= 1
+                c("} else {")
+                c.ind += 1
+            for e in range(sp.n):
+                c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
+            if self.pair_access():
+                c.ind -= 1
+                c("}")
             if sp.BS > 1:
                 c.ind -= 1
                 c("} else {")
@@ -480,11 +489,18 @@ class KernelEmitter:
                 c("if ((row0 + s) < a.nrows) {")
                 c.ind += 1
             if self.pair_access():
+                c("if (((unsigned long long)out & 15ull) == 0ull) {")
+                c.ind += 1
                 for e in range(0, sp.n, 2):
                     c(f"{self.GST}2(out, ubase, {e}, go, r[{self.out_reg(e)}], r[{self.out_reg(e + 1)}]);")
-            else:
-                for e in range(sp.n):
-                    c(f"{self.GST}(out, ubase, {sp.Tr * e}, go, r[{self.out_reg(e)}]);")
+                c.ind -= 1
+                c("} else {")
+                c.ind += 1
+            for e in range(sp.n):
+                c(f"{self.GST}(out, ubase, {sp.Tr * e}, go, r[{self.out_reg(e)}]);")
+            if self.pair_access():
+                c.ind -= 1
+                c("}")
             if sp.BS > 1:
                 c.ind -= 1
                 c("}")

@@ -49,7 +49,7 @@ __device__ __forceinline__ void tfft_bst(double2* p, unsigned voff, unsigned sof
 }
 // Two adjacent fp32 elements in one 128-bit access: for kernels whose threads hold whole
 // transforms, so that a lane's elements are contiguous.  The byte address must be a multiple
-// of 16 (the host checks the tensor pointers of plans that use these).
+// of 16: the kernels test the tensor pointer and use the one-element accesses otherwise.
 template <int AUX = 0>
 __device__ __forceinline__ void tfft_bld2(const float2* p, unsigned voff, unsigned soff, float2& a, float2& b) {
     const tfft_u4 t = __builtin_amdgcn_raw_buffer_load_b128(tfft_rsrc(p), voff, soff, AUX);
