@@ -357,6 +357,26 @@ def test_whole_transform_threads_take_any_buffer_alignment():
         plan.close()
 
 
+def test_tuned_tiles_per_block_shrink_with_the_batch():
+    # fp32 2^15 walks 16 tiles per block in the built-in table, tuned with the device full: a
+    # batch with fewer tiles than that per resident block slot gets a block per tile (or as many
+    # tiles per block as leave one block per slot), and the result is the same transform
+    torch = _torch()
+    for logN, tiles in ((15, 16),):
+        N = 1 << logN
+        plan = turbofft_amd.TurboFFT(logN, "float2")
+        slots = plan.tb_gap(0)
+        assert plan.grid(0, 7) == 7 and plan.grid(0, slots) == slots
+        assert plan.grid(0, 3 * slots) == slots
+        assert plan.grid(0, tiles * slots * 2) == 2 * slots
+        for bs in (7, 3 * slots + 5):
+            xh = make(bs, N, "float2", logN + bs)
+            y = plan.fft(torch.from_numpy(xh).cuda()).cpu().numpy()
+            sel = np.unique(np.linspace(0, bs - 1, 9).astype(int))
+            assert O.rel_l2(y[sel], O.fft_ref(xh[sel])) <= O.tolerance("float2", logN)
+        plan.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT

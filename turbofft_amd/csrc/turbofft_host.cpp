@@ -186,6 +186,7 @@ struct c64 { double x, y; };
 
 struct turbofft_plan {
     int logN = 0, datatype = 0, if_ft = 0, if_err = 0, thread_bs = 1;
+    bool tiles_from_row = false;   // thread_bs is the plan row's tuned tiles-per-block, not the caller's
     Row row{};
     int launches = 0;
     const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
@@ -310,7 +311,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     // leaves thread_bs at its default gets the value tuned for this size (large tiles amortise
     // the block launch over several of them).  With fault tolerance thread_bs is the checksum
     // group size and stays what the caller asked for.
-    if (!p->if_ft && p->thread_bs == 1 && r.tiles() > 1) p->thread_bs = r.tiles();
+    if (!p->if_ft && p->thread_bs == 1 && r.tiles() > 1) { p->thread_bs = r.tiles(); p->tiles_from_row = true; }
     int sum = 0;
     for (int i = 0; i < p->launches; ++i) sum += r.logNi(i);
     if (sum != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row for logN=%d: digit sizes sum to %d", p->logN, sum);
@@ -464,10 +465,20 @@ static long long launch_tiles(const turbofft_plan* p, int i, long long bs) {
     return pts / tile;
 }
 
+// Tiles a block of launch i walks.  The row's tuned value was timed with the device full: a
+// batch too small for that keeps at least one block per resident slot instead.
+static int launch_thread_bs(const turbofft_plan* p, int i, long long ntiles) {
+    if (!p->tiles_from_row) return p->thread_bs;
+    long long per_slot = ntiles / (p->resident[i] > 0 ? p->resident[i] : 1);
+    if (per_slot < 1) per_slot = 1;
+    return per_slot < p->thread_bs ? (int)per_slot : p->thread_bs;
+}
+
 long long turbofft_plan_grid(const turbofft_plan_t* p, int launch, long long bs) {
     if (!p || launch < 0 || launch >= p->launches || bs < 0) return fail(TURBOFFT_EINVAL, "bad argument");
     long long nt = launch_tiles(p, launch, bs);
-    return (nt + p->thread_bs - 1) / p->thread_bs;
+    int tbs = launch_thread_bs(p, launch, nt);
+    return (nt + tbs - 1) / tbs;
 }
 
 int turbofft_plan_tb_gap(const turbofft_plan_t* p, int launch) {
@@ -579,7 +590,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         memset(&a, 0, sizeof a);
         a.ntiles = launch_tiles(p, i, bs);
         a.nrows = bs;
-        a.thread_bs = p->thread_bs;
+        a.thread_bs = launch_thread_bs(p, i, a.ntiles);
         a.tb_gap = p->tb_gap[i];
         if (k->pf && !p->if_ft && p->thread_bs == 1 && a.ntiles > p->resident[i]) {
             // prefetching kernels run as a persistent grid: one block per resident slot walks
