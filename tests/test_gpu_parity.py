@@ -377,6 +377,35 @@ def test_tuned_tiles_per_block_shrink_with_the_batch():
         plan.close()
 
 
+@pytest.mark.parametrize("dt,logN,log_bs", [("float2", 13, 19), ("float2", 20, 11), ("double2", 17, 14)])
+def test_data_sets_beyond_4_gib(dt, logN, log_bs):
+    # 2^31 and 2^32 points (16 and 32 GiB in): element offsets pass 2^32, byte offsets 2^35.
+    # Sampled transforms (first, last, around the middle, six seeded) against the oracle, and
+    # Parseval over every transform of the batch
+    torch = _torch()
+    N, bs = 1 << logN, 1 << log_bs
+    x = torch.empty((bs, N), dtype=torch.complex64 if dt == "float2" else torch.complex128, device="cuda")
+    xr = torch.view_as_real(x)
+    step = bs // 64
+    g = torch.Generator(device="cuda").manual_seed(logN)
+    for b0 in range(0, bs, step):       # in slices, to bound the temporaries
+        xr[b0:b0 + step].uniform_(-1, 1, generator=g)
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    out = torch.empty(plan.out_elems(bs), dtype=x.dtype, device="cuda")
+    plan.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    y = out[: bs * N].view(bs, N)
+    rows = sorted({0, 1, bs // 2 - 1, bs // 2, bs - 2, bs - 1} | {int(v) for v in np.random.default_rng(1).integers(0, bs, 6)})
+    for r in rows:
+        assert O.rel_l2(y[r].cpu().numpy()[None], O.fft_ref(x[r].cpu().numpy()[None])) <= O.tolerance(dt, logN), r
+    num = sum(float((y[b0:b0 + step].abs().double() ** 2).sum()) for b0 in range(0, bs, step))
+    den = sum(float((x[b0:b0 + step].abs().double() ** 2).sum()) for b0 in range(0, bs, step))
+    assert abs(num / den / N - 1) < (1e-5 if dt == "float2" else 1e-12)
+    plan.close()
+    del x, xr, out, y
+    torch.cuda.empty_cache()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT
