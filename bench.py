@@ -10,7 +10,8 @@ whole batch.  Prints ONE JSON line:
   roofline     : dominant kernel against the 8 TB/s HBM peak, timed with HIP
                  events on the launch stream over the timed region
   cpu_baseline : scipy.fft (pocketfft) on the host cores for a bounded sample
-                 of the same workload, scaled to the same unit
+                 of the same workload, scaled to the same unit; "single_thread" inside it
+                 is numpy.fft.fft, the routine of the accuracy oracle, on one core
   ft_overhead  : run time of the same workload with the fused checksums over the
                  plain plan, measured after the timed region (--no_ft_overhead skips it);
                  "offline" inside it is the same comparison for separate checksum passes
@@ -132,10 +133,24 @@ def cpu_baseline(logN, datatype, target_s=10.0):
     pts = calls * nb * N
     esize = 8 if datatype == 0 else 16
     gbs = 2 * pts * esize / el / 1e9
+    # the routine the accuracy oracle itself calls (numpy's pocketfft, one thread), for ~3 s
+    np.fft.fft(x, axis=-1)
+    t1 = time.perf_counter()
+    calls1 = 0
+    while True:
+        np.fft.fft(x, axis=-1)
+        calls1 += 1
+        el1 = time.perf_counter() - t1
+        if el1 >= min(3.0, target_s) or calls1 >= 1000000:
+            break
+    pts1 = calls1 * nb * N
     return {"value": gbs, "unit": "GB/s", "cores": cores, "kind": "port",
             "gflops": 5.0 * pts * logN / el / 1e9,
             "sample": f"scipy.fft.fft (pocketfft, workers={cores}) on {calls} x ({nb} x 2^{logN}) "
-                      f"{'complex64' if datatype == 0 else 'complex128'} transforms, {el:.1f} s"}
+                      f"{'complex64' if datatype == 0 else 'complex128'} transforms, {el:.1f} s",
+            "single_thread": {"value": 2 * pts1 * esize / el1 / 1e9, "unit": "GB/s", "cores": 1,
+                              "gflops": 5.0 * pts1 * logN / el1 / 1e9,
+                              "sample": f"numpy.fft.fft on {calls1} x ({nb} x 2^{logN}) transforms, {el1:.1f} s"}}
 
 
 def main():
