@@ -406,6 +406,38 @@ def test_data_sets_beyond_4_gib(dt, logN, log_bs):
     torch.cuda.empty_cache()
 
 
+def test_plans_on_concurrent_streams():
+    # independent plans (and one plain plan shared by two streams: it owns no scratch memory)
+    # queued on different streams at the same time give the results of running them one by one
+    torch = _torch()
+    cases = [("float2", 13, 600), ("double2", 16, 40), ("float2", 20, 6), ("double2", 9, 5000)]
+    xs = [torch.from_numpy(make(bs, 1 << logN, dt, logN)).cuda() for dt, logN, bs in cases]
+    plans = [turbofft_amd.TurboFFT(logN, dt) for dt, logN, bs in cases]
+    outs = [torch.zeros(p.out_elems(bs), dtype=x.dtype, device="cuda") for p, x, (dt, logN, bs) in zip(plans, xs, cases)]
+    ref = [p.fft(x).clone() for p, x in zip(plans, xs)]
+    streams = [torch.cuda.Stream() for _ in cases]
+    torch.cuda.synchronize()
+    for rep in range(5):
+        for p, x, o, st, (dt, logN, bs) in zip(plans, xs, outs, streams, cases):
+            p.exec(x.data_ptr(), o.data_ptr(), bs, st.cuda_stream)
+    torch.cuda.synchronize()
+    for o, r in zip(outs, ref):
+        assert torch.equal(o[: r.numel()].view_as(r), r)
+    # one plain single-launch plan on two streams, different buffers
+    p, x, (dt, logN, bs) = plans[0], xs[0], cases[0]
+    x2 = torch.from_numpy(make(bs, 1 << logN, dt, 99)).cuda()
+    r2 = p.fft(x2).clone()
+    o1, o2 = torch.zeros_like(ref[0]), torch.zeros_like(r2)
+    torch.cuda.synchronize()
+    for rep in range(5):
+        p.exec(x.data_ptr(), o1.data_ptr(), bs, streams[0].cuda_stream)
+        p.exec(x2.data_ptr(), o2.data_ptr(), bs, streams[1].cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, ref[0]) and torch.equal(o2, r2)
+    for p in plans:
+        p.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT
