@@ -61,7 +61,7 @@ def test_builtin_rows_match_csv_and_are_consistent(dtype):
 
 def test_optional_plan_columns():
     """Columns beyond the reference's 11: per-launch split / prefetch / cross-lane flags,
-    tiles per block, per-launch wavefronts per SIMD, per-launch non-temporal accesses.
+    tiles per block, per-launch wavefronts per SIMD, per-launch tile access policy.
     Shorter rows mean zeros."""
     from turbofft_amd.codegen.fft_codegen import generate_source
     r = P.PlanRow.from_list([19, 2, 9, 10, 0, 32, 16, 0, 32, 32, 0, 1, 1, 0, 0, 0, 0, 0, 0, 0, 8, 4, 3])
@@ -79,8 +79,16 @@ def test_optional_plan_columns():
     assert [k.name for k in P.kernels_for_row(r, "float2", 1)] == ["tfft_f32_col_N9_b32_n32_t3_ft", "tfft_f32_rowT_N10_b16_n32_t2_ft"]
     src = generate_source([KernelSpec(P.kernels_for_row(r, "float2", 0)[1])], False)
     assert "GLDG(" in src and "GSTGN(" in src and "GLDGN(" not in src and "GSTG(" not in src
+    # +4 in the same columns: the wave raises its priority while it issues its tile loads
+    # (plain single-launch kernels; the fault-tolerant flavour of the row drops the bit)
+    r = P.PlanRow.from_list([12, 1, 12, 0, 0, 1, 0, 0, 16, 0, 0] + [0] * 13 + [7])
+    assert [k.name for k in P.kernels_for_row(r, "float2", 0)] == ["tfft_f32_row1_N12_b1_n16_t7"]
+    assert [k.name for k in P.kernels_for_row(r, "float2", 1)] == ["tfft_f32_row1_N12_b1_n16_t3_ft"]
+    src = generate_source([KernelSpec(P.kernels_for_row(r, "float2", 0)[0])], False)
+    assert src.index("TFFT_WAVE_PRIO(3);") < src.index("GLDUN(") < src.index("TFFT_WAVE_PRIO(0);") < src.index("cadd(")
+    assert "TFFT_WAVE_PRIO" not in generate_source([KernelSpec(P.kernels_for_row(r, "float2", 1)[0])], False)
     with pytest.raises(ValueError):
-        P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0] + [0] * 13 + [4])
+        P.PlanRow.from_list([13, 1, 13, 0, 0, 1, 0, 0, 32, 0, 0] + [0] * 13 + [8])
     # columns 28-30: tiles per XCD, a launch parameter (no kernel depends on it)
     r = P.PlanRow.from_list([20, 2, 10, 10, 0, 16, 16, 0, 32, 32, 0] + [0] * 16 + [8, 32])
     assert r.xc == (8, 32)

@@ -36,7 +36,7 @@ class PlanRow:
     xl: Tuple[int, ...] = ()         # optional columns 18-20: 1 = last small-radix pass across lanes
     tiles: int = 0                   # optional column 21: tiles per block of the plain plan (0 = 1)
     wv: Tuple[int, ...] = ()         # optional columns 22-24: wavefronts per SIMD to compile for (0 = free)
-    nt: Tuple[int, ...] = ()         # optional columns 25-27: 1 = non-temporal tile loads, 2 = stores, 3 = both
+    nt: Tuple[int, ...] = ()         # optional columns 25-27, tile access policy: +1 non-temporal tile loads, +2 non-temporal stores, +4 raised wave priority while the loads are issued
     xc: Tuple[int, ...] = ()         # optional columns 28-30: consecutive tiles per XCD (run time only; 0 = 64)
 
     @staticmethod
@@ -53,8 +53,8 @@ class PlanRow:
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
                     tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
                     tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]), tuple((row[27:30] + [0, 0, 0])[:L]))
-        if any(t not in (0, 1, 2, 3) for t in p.nt):
-            raise ValueError(f"non-temporal columns must be 0..3 in row {row}")
+        if any(t not in range(8) for t in p.nt):
+            raise ValueError(f"tile access policy columns must be 0..7 in row {row}")
         if L and sum(p.logNi) != p.logN:
             raise ValueError(f"logN1+logN2+logN3 != logN in row {row}")
         return p
@@ -76,7 +76,7 @@ class KernelKey:
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
     wv: int = 0      # > 0: compiled to fit this many wavefronts per SIMD (register budget 512 / wv)
-    nt: int = 0      # bit 0: tile loads are non-temporal, bit 1: tile stores are
+    nt: int = 0      # bit 0: tile loads are non-temporal, bit 1: tile stores are, bit 2: raised wave priority while the tile loads are issued (plain kernels)
     inv: int = 0     # 1: the flavour an inverse plan uses in this position -- re and im exchanged as
                      # they are loaded (row1, col as first launch) and/or before they are stored
                      # (row1, rowT): inverse = swap . forward . swap
@@ -117,7 +117,8 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False) ->
                       # the register budget hint was tuned on the plain kernel only (fault-tolerant
                       # kernels keep their table in registers and spill under any tighter budget)
                       (int(row.wv[i]) if row.wv else 0) if not ft else 0,
-                      int(row.nt[i]) if row.nt else 0,
+                      # the priority bit was timed on the plain kernel only
+                      (int(row.nt[i]) & (3 if ft else 7)) if row.nt else 0,
                       1 if inverse and i in (0, last) else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 

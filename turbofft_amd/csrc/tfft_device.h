@@ -60,6 +60,8 @@ __device__ __forceinline__ void tfft_bst2(float2* p, unsigned voff, unsigned sof
     tfft_u4 t; t.x = __float_as_uint(a.x); t.y = __float_as_uint(a.y); t.z = __float_as_uint(b.x); t.w = __float_as_uint(b.y);
     __builtin_amdgcn_raw_buffer_store_b128(t, tfft_rsrc(p), voff, soff, AUX);
 }
+// priority of the calling wave for instruction issue on its SIMD (0 lowest, 3 highest)
+#define TFFT_WAVE_PRIO(n) __builtin_amdgcn_s_setprio(n)
 #define TFFT_ESZ(p) ((unsigned)sizeof(*(p)))
 #define GLDU2(p, ub, uo, off, A, B) tfft_bld2<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
 #define GSTU2(p, ub, uo, off, A, B) tfft_bst2<0>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (A), (B))
@@ -125,6 +127,7 @@ extern long long tfft_sim_errors;
 #define GSTUN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
 #define GLDGN(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTGN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
+#define TFFT_WAVE_PRIO(n) ((void)0)
 #define GLDU2(p, ub, uo, off, A, B) { (A) = GLDU(p, ub, uo, off); (B) = GLDU(p, ub, (uo) + 1, off); }
 #define GSTU2(p, ub, uo, off, A, B) { GSTU(p, ub, uo, off, A); GSTU(p, ub, (uo) + 1, off, B); }
 #define GLDUN2(p, ub, uo, off, A, B) GLDU2(p, ub, uo, off, A, B)

@@ -15,7 +15,7 @@ typedef struct tfft_kernel_entry {
     int pf;              // 1: the block prefetches its next tile (wants a persistent grid)
     int xl;              // 1: the last small-radix pass runs across lanes (DPP / ds_swizzle)
     int wv;              // > 0: compiled for this many wavefronts per SIMD
-    int nt;              // bit 0: non-temporal tile loads, bit 1: non-temporal tile stores
+    int nt;              // bit 0: non-temporal tile loads, bit 1: non-temporal tile stores, bit 2: raised wave priority for the tile loads
     int inv;             // 1: component-swapping flavour for the first / last launch of an inverse plan
     int threads;         // block size
     int lds_bytes;       // dynamic LDS

@@ -327,7 +327,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
         int kind = kind_of_launch(p->launches, i);
         const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
                                                  (r.xl(i) && !p->if_ft) ? 1 : 0,    // FT plans keep the LDS path
-                                                 p->if_ft ? 0 : r.wv(i), r.nt(i));
+                                                 p->if_ft ? 0 : r.wv(i), p->if_ft ? (r.nt(i) & 3) : r.nt(i));   // wave budget and priority bit: plain kernels only
         if (!k)
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
