@@ -729,7 +729,7 @@ class KernelEmitter:
                     # A wave that is about to fetch its tile goes first: the loads of a block that
                     # has just started are issued before the arithmetic of the blocks already
                     # resident gets the slot.  Measured per size; a policy bit of the plan row.
-                    prio = bool(int(sp.key.nt) & 4) and sp.kind == "row1"
+                    prio = bool(int(sp.key.nt) & 4)
                     if prio:
                         c("TFFT_WAVE_PRIO(3);")
                     self.emit_load(c)
