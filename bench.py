@@ -13,9 +13,13 @@ whole batch.  Prints ONE JSON line:
                  of the same workload, scaled to the same unit; "single_thread" inside it
                  is numpy.fft.fft, the routine of the accuracy oracle, on one core
   ft_overhead  : run time of the same workload with the fused checksums over the
-                 plain plan, measured after the timed region (--no_ft_overhead skips it);
+                 plain plan, measured after the timed region in alternating blocks
+                 (plain, checksummed, plain, ...) so that both see the same device state;
+                 the ratio of the two medians (--no_ft_overhead skips it);
                  "offline" inside it is the same comparison for separate checksum passes
                  before and after the plain plan (the reference's cufft_ft.h baseline)
+  prewarm_s    : untimed executions before the warm-up steps, by time rather than by count:
+                 a device that has been idle clocks up over its first tenths of a second
   vendor_baseline : hipFFT (rocFFT) on the same buffers and workload, after the timed
                  region, the side-by-side the reference runs against cuFFT
                  (main.cu:105,121); --no_vendor skips it
@@ -52,10 +56,31 @@ def make_input(torch, bs, N, datatype, seed=0):
     return torch.view_as_complex(x)
 
 
+def prewarm(torch, plan, x, out, bs, seconds):
+    """Keep the device busy with the workload for `seconds` (untimed, not part of the steps)."""
+    stream = torch.cuda.current_stream().cuda_stream
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+        n += 8
+        torch.cuda.synchronize()
+    return time.perf_counter() - t0, n
+
+
+def stats(v):
+    v = sorted(v)
+    return {"mean": sum(v) / len(v), "min": v[0], "median": v[len(v) // 2] if len(v) % 2 else 0.5 * (v[len(v) // 2 - 1] + v[len(v) // 2]),
+            "max": v[-1]}
+
+
 def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if_err=0, thread_bs=1, param=None,
-             x=None, out=None):
+             x=None, out=None, prewarm_s=0.0, correct=None):
     N = 1 << logN
     plan = turbofft_amd.TurboFFT(logN, datatype, if_ft=if_ft, if_err=if_err, thread_bs=thread_bs, param_csv=param)
+    if correct is not None:
+        plan.set_ft_params(1000.0, 1e-3, correct)
     cdt = torch.complex64 if datatype == 0 else torch.complex128
     if x is None:
         x = make_input(torch, bs, N, datatype)
@@ -65,33 +90,70 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
         raise ValueError(f"buffers too small for logN={logN} bs={bs}: out holds {out.numel()} elements, "
                          f"the plan needs {plan.out_elems(bs)}")
     stream = torch.cuda.current_stream().cuda_stream
+    pre_s, pre_n = prewarm(torch, plan, x, out, bs, prewarm_s) if prewarm_s > 0 else (0.0, 0)
     for _ in range(warmup):
         plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
     torch.cuda.synchronize()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
+    # one event between every two steps (on the stream the kernels are launched on): the whole
+    # region gives the mean, the intervals its spread
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(steps):
+    ev[0].record()
+    for i in range(steps):
         plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
-    ev1.record()
+        ev[i + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     wall_ms = (t1 - t0) * 1000.0 / steps
-    ev_ms = ev0.elapsed_time(ev1) / steps
+    ev_ms = ev[0].elapsed_time(ev[steps]) / steps
+    per_step = [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
     res = {
         "logN": logN, "datatype": datatype, "bs": bs, "launches": plan.launches,
         "plan": {"logNi": plan.logNi, "BS": plan.BS, "n": plan.n, "threads": plan.threads, "lds_bytes": plan.lds_bytes},
-        "wall_ms": wall_ms, "event_ms": ev_ms,
+        "wall_ms": wall_ms, "event_ms": ev_ms, "step_ms": stats(per_step),
         "gbs": plan.gbs(bs, wall_ms), "gflops": plan.gflops(bs, wall_ms),
-        "alg_bytes": plan.algorithmic_bytes(bs),
+        "alg_bytes": plan.algorithmic_bytes(bs), "prewarm_s": pre_s, "prewarm_execs": pre_n,
     }
     if if_ft or if_err:
         # counters accumulate over every execution of the plan (warm-up included)
-        res["ft"] = {k: v for k, v in plan.ft_counters().items() if k != "flagged"}
-        res["ft"]["execs"] = warmup + steps
+        res["ft"] = {k: v for k, v in plan.ft_counters().items() if k not in ("flagged", "flagged_truncated")}
+        res["ft"]["execs"] = pre_n + warmup + steps
     plan.close()
     return res, x, out
+
+
+def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param, thread_bs=4, rounds=7, block=10):
+    """Plain and checksummed plan of the same workload in alternating blocks of `block`
+    executions (plain first and last), each block between two events; the overhead is the
+    ratio of the median block times, so neither plan is measured on a colder device."""
+    plain = turbofft_amd.TurboFFT(logN, datatype, param_csv=param)
+    ft = turbofft_amd.TurboFFT(logN, datatype, if_ft=1, thread_bs=thread_bs, param_csv=param)
+    stream = torch.cuda.current_stream().cuda_stream
+    for pl in (plain, ft):
+        for _ in range(3):
+            pl.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+    torch.cuda.synchronize()
+    times = {0: [], 1: []}
+    marks = []
+    for r in range(2 * rounds + 1):
+        which = r % 2
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(block):
+            (ft if which else plain).exec(x.data_ptr(), out.data_ptr(), bs, stream)
+        e1.record()
+        marks.append((which, e0, e1))
+    torch.cuda.synchronize()
+    for which, e0, e1 in marks:
+        times[which].append(e0.elapsed_time(e1) / block)
+    counters = {k: v for k, v in ft.ft_counters().items() if k not in ("flagged", "flagged_truncated")}
+    info = {"logNi": ft.logNi, "BS": ft.BS, "n": ft.n, "threads": ft.threads, "lds_bytes": ft.lds_bytes}
+    plain.close()
+    ft.close()
+    p, f = stats(times[0]), stats(times[1])
+    return {"overhead_pct": 100.0 * (f["median"] / p["median"] - 1.0), "plain_ms": p, "ft_ms": f, "ms_per_step": f["median"],
+            "thread_bs": thread_bs, "order": "plain/ft alternating, %d blocks of %d executions each" % (2 * rounds + 1, block),
+            "plan": info, "counters": counters}
 
 
 def vendor_case(torch, turbofft_amd, logN, datatype, bs, x, out, reps=20, warmup=2):
@@ -165,6 +227,9 @@ def main():
     ap.add_argument("--if_err", type=int, default=0)
     ap.add_argument("--thread_bs", type=int, default=1)
     ap.add_argument("--param", type=str, default=None)
+    ap.add_argument("--prewarm_s", type=float, default=1.0,
+                    help="seconds of untimed executions before the warm-up steps (reported as prewarm_s)")
+    ap.add_argument("--correct", type=int, default=None, help="with --if_err: 1 recompute, 2 delayed batch correction")
     ap.add_argument("--no_cpu", action="store_true")
     ap.add_argument("--cpu_seconds", type=float, default=10.0)
     ap.add_argument("--sweep", action="store_true")
@@ -203,7 +268,7 @@ def main():
                     x = x.view(-1).view(bs, 1 << logN)
                 try:
                     r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err,
-                                         a.thread_bs, a.param, x, out)
+                                         a.thread_bs, a.param, x, out, prewarm_s=min(a.prewarm_s, 0.2), correct=a.correct)
                 except turbofft_amd.TurboFFTError as e:
                     # a plan row without a compiled kernel must not stop the sweep; anything
                     # that comes from the device does
@@ -213,7 +278,7 @@ def main():
                 if "gbs" in r:
                     r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
                     print(f"{'fp32' if dt == 0 else 'fp64'} logN={logN:2d} L={r['launches']} "
-                          f"{r['wall_ms']:8.3f} ms {r['gflops']:9.1f} GFLOPS {r['gbs']:8.1f} GB/s  "
+                          f"{r['wall_ms']:8.3f} ms (min {r['step_ms']['min']:.3f}) {r['gflops']:9.1f} GFLOPS {r['gbs']:8.1f} GB/s  "
                           f"{100 * r['frac_hbm']:5.1f}% of HBM peak  {r['plan']}"
                           + (f"  ft per exec: " + " ".join(f"{k} {v // r['ft']['execs']}" for k, v in r["ft"].items() if k != "execs")
                              if "ft" in r else ""), flush=True)
@@ -243,7 +308,8 @@ def main():
 
     logN, dt = a.logN, a.datatype
     bs = a.bs or (1 << (28 - logN))
-    r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err, a.thread_bs, a.param)
+    r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err, a.thread_bs, a.param,
+                         prewarm_s=a.prewarm_s, correct=a.correct)
     for _ in range(a.calib_copy):
         out.view(-1)[: x.numel()].copy_(x.view(-1))          # reads and writes x.numel()*sizeof(T) bytes
     torch.cuda.synchronize()
@@ -251,17 +317,20 @@ def main():
     if not (a.if_ft or a.if_err) and not a.no_ft_overhead:
         # the second half of the headline metric: the same workload with the fused checksums
         # (4 tiles per checksum group, no error injected), outside the timed region above
-        rf, x, out = run_case(torch, turbofft_amd, logN, dt, bs, max(20, a.steps // 4), min(a.warmup, 5), 1, 0, 4,
-                              a.param, x, out)
-        ft_line = {"overhead_pct": 100.0 * (rf["event_ms"] / r["event_ms"] - 1.0), "ms_per_step": rf["wall_ms"],
-                   "thread_bs": 4, "plan": rf["plan"], "counters": rf.get("ft")}
+        ft_line = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param)
         # the offline scheme on the same workload: checksum pass, plain plan, checksum pass, compare
         try:
             oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 10),
                                                       torch.cuda.current_stream().cuda_stream)
-            ft_line["offline"] = {"overhead_pct": 100.0 * (oms / r["event_ms"] - 1.0), "ms_per_step": oms, "flagged": oflag}
+            ft_line["offline"] = {"overhead_pct": 100.0 * (oms / ft_line["plain_ms"]["median"] - 1.0), "ms_per_step": oms, "flagged": oflag}
         except turbofft_amd.TurboFFTError as e:
             ft_line["offline"] = {"error": str(e)}
+    sync_ms = None
+    if not (a.if_ft or a.if_err):
+        # the reference's own timing protocol beside the default one: a host wait after every launch
+        pl = turbofft_amd.TurboFFT(logN, dt, param_csv=a.param)
+        sync_ms = pl.time_sync(x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 4), torch.cuda.current_stream().cuda_stream)
+        pl.close()
     vendor_line = None
     if not a.no_vendor:
         vendor_line = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(10, a.steps // 10))
@@ -275,7 +344,7 @@ def main():
     line = {
         "metric": "batched C2C FFT algorithmic HBM GB/s (2*N*bs*sizeof(T)/t) at logBS+logN=28",
         "value": r["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": r["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": r["wall_ms"], "step_ms": r["step_ms"], "prewarm_s": r["prewarm_s"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if dt == 0 else "f64", "data": "synthetic",
         "gflops": r["gflops"],
         "config": {"workload": f"forward C2C FFT {tname} N=2^{logN} batch=2^{int(math.log2(bs))} "
@@ -287,6 +356,8 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get((dt, logN, bs, int(bool(a.if_ft or a.if_err)))),
                      "kernel_ms": kernel_ms, "alg_bytes_per_launch": r["alg_bytes"]},
     }
+    if sync_ms is not None:
+        line["ms_per_step_sync_each_launch"] = sync_ms          # main.cu:53-62 protocol, reported only
     if a.if_ft or a.if_err:
         line["ft"] = r.get("ft")
     if ft_line is not None:

@@ -16,7 +16,8 @@
  * batch-major x[b*N + n]; the result is out-of-place, natural order, same
  * shape.  `in` is never written.  When the plan uses more than one launch
  * `out` must hold 2*N*bs elements (initializeData.h:21, main.cu:11-12); the
- * transform is left in out[0 .. N*bs), the second half is workspace.
+ * transform is left in out[0 .. N*bs), the second half is workspace.  `in`
+ * must not overlap `out` (workspace included): TURBOFFT_EINVAL otherwise.
  */
 #ifndef TURBOFFT_H
 #define TURBOFFT_H
@@ -97,6 +98,12 @@ int turbofft_exec_host(turbofft_plan_t* plan, const void* in_h, void* out_h, lon
 int turbofft_time(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
                   int warmup, int reps, void* stream, float* ms_per_exec);
 
+/* The reference's own timing protocol: as turbofft_time, but the host waits for every launch
+ * before issuing the next and once more after each execution (main.cu:53-62), so launch
+ * latency and the idle device between launches are part of the figure. */
+int turbofft_time_sync(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
+                       int warmup, int reps, void* stream, float* ms_per_exec);
+
 /* Like turbofft_time, with HIP events around every launch of the plan:
  * ms_per_launch[i] receives the mean duration of launch i (entries beyond the
  * plan's launch count are set to 0).  No counterpart in the reference, which
@@ -121,8 +128,27 @@ int turbofft_plan_set_tb_gap(turbofft_plan_t* plan, int launch, int tb_gap);
 /* ---- fault tolerance (no counterpart API in the reference; its generator
  * bakes these into the kernel text: fft_codegen.py:412-415, 495, 714-719) ---- */
 
-/* Detection rule |delta| / (err_smoothing + |mag|) > err_threshold. */
+/* Detection rule |delta| / (err_smoothing + |mag|) > err_threshold, and what happens to a
+ * located tile:
+ *   correct 0  detect and report only
+ *   correct 1  recompute the tile from its input (the correction the reference's if_err=1
+ *              kernels run, fft_codegen.py:149-193); the result is bit-identical to an
+ *              undisturbed run
+ *   correct 2  delayed batch correction: every thread keeps the sums of the inputs and of the
+ *              outputs of its group's tiles (the live sums of fft_codegen.py:355-357,421-423)
+ *              and the located tile is patched in place with FFT(sum x) - sum y (the lines
+ *              commented at fft_codegen.py:401-404,427-429; test.ipynb cell 0).  The tile's
+ *              input is not read again; the patched result equals the undisturbed one to
+ *              rounding, not bit for bit.  Kernels of this flavour are built for the built-in
+ *              fault-tolerant plan rows; TURBOFFT_ENOPLAN otherwise. */
 int turbofft_set_ft_params(turbofft_plan_t* plan, double err_smoothing, double err_threshold, int correct);
+
+/* Which checksum table the plan's kernels read: 0 = exact angles (the default), 1 = the
+ * reference's own table, whose angles 2*pi*i*j are rounded to float before the division by N
+ * (abft.h:34-35,55-56, built at main.cu:85-93).  Waits for the plan's last execution, then
+ * replaces the tables.  The environment variable TURBOFFT_CHECKSUM_MODE=1 selects mode 1 at
+ * plan creation. */
+int turbofft_set_checksum_mode(turbofft_plan_t* plan, int mode);
 
 /* Error injection for the launch `launch` (-1 = last, the reference's choice):
  *   mode 0  none
@@ -134,10 +160,14 @@ int turbofft_set_ft_params(turbofft_plan_t* plan, double err_smoothing, double e
 int turbofft_set_injection(turbofft_plan_t* plan, int mode, int launch, int every,
                            long long tile_phase, int s, int m, double mag);
 
-/* Counters accumulated since the last reset: groups checked, detected,
- * corrected, uncorrectable (located tile out of range); flagged[2*i] = launch,
- * flagged[2*i+1] = tile (-1 if not locatable), up to `cap` pairs; *nflagged
- * receives the number recorded.  Synchronises the device. */
+/* Counters accumulated since the last reset: groups checked, detected, corrected,
+ * uncorrectable (located tile out of range); flagged[2*i] = launch, flagged[2*i+1] = tile
+ * (-1 if not locatable), up to `cap` pairs; *nflagged receives the number written.  The
+ * plan records at most 4096 pairs between resets: the list is truncated when *detected
+ * exceeds *nflagged.  All four counters live on the device (`checked` is added by the first
+ * block of every launch), so replays of a captured HIP graph are counted.  Waits for the
+ * stream of the plan's most recent turbofft_exec only, not for the device: work the caller
+ * put on other streams (a graph replayed elsewhere) has to be synchronised by the caller. */
 int turbofft_get_ft_counters(turbofft_plan_t* plan, unsigned long long* checked,
                              unsigned long long* detected, unsigned long long* corrected,
                              unsigned long long* uncorrectable, long long* flagged, int cap,

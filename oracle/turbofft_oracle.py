@@ -18,6 +18,11 @@ Parity status (what pins each function):
   block_fft / plan_fft    restatement of the reference kernel algebra (DIF
                           passes, twiddle recurrences, four-step digit maps);
                           checked against fft_ref for every plan class.
+  delayed_batch_correction  the reference's batch-sum correction (live sums, commented
+                          correction lines, notebook algebra); pinned by linearity: the
+                          patched tile must equal the clean transform for errors of any
+                          shape on one tile, and a flipped sign, a dropped sum or a wrong
+                          tile index leaves an error of the injected size.
   ft_launch_model         restatement of the reference checksum arithmetic;
                           checked against the closed-form checksum shift of an
                           injected error and the "clean data -> no detection"
@@ -574,6 +579,30 @@ def ft_launch_model(xin: np.ndarray, yout: np.ndarray, n: int, groups: List[List
                 tile = tiles[k - 1]
         out.append(GroupDecision(delta, delta2, mag, bool(det), k, tile))
     return out
+
+
+def delayed_batch_correction(x_tiles: np.ndarray, y_tiles: np.ndarray, k: int, n: int, dtype) -> np.ndarray:
+    """Delayed batch correction of one checksum group (fft_codegen.py:355-357 per-thread input
+    sums, :421-423 output sums, the correction lines commented at :401-404 and :427-429, and
+    the algebra of test.ipynb cell 0 with unit weights):
+
+        y_k  <-  y_k + FFT(sum_t x_t) - sum_t y_t
+
+    x_tiles[t, s, m] are the inputs of the group's tiles in processing order, y_tiles[t, s, j]
+    the outputs as the kernel produced them (tile k, 0-based, carrying the error), both before
+    any inter-launch twiddle.  Sums run over t in order, in T; the transform of the summed
+    input is the in-block FFT in T.  By linearity the patched tile equals the clean
+    transform of x_k when no other tile of the group is corrupted; unlike a recompute it is
+    not bit-identical to it (its rounding error grows with the group size).
+    Returns the patched y_tiles[k]."""
+    ct = _ctype(dtype)
+    sx = np.zeros(x_tiles.shape[1:], ct)
+    sy = np.zeros(y_tiles.shape[1:], ct)
+    for t in range(x_tiles.shape[0]):
+        sx = (sx + x_tiles[t].astype(ct)).astype(ct)
+        sy = (sy + y_tiles[t].astype(ct)).astype(ct)
+    corr = (block_fft(sx, n, dtype) - sy).astype(ct)
+    return (y_tiles[k].astype(ct) + corr).astype(ct)
 
 
 def injected_delta_closed_form(Ni: int, mag: float) -> float:

@@ -18,8 +18,8 @@ def rnd(shape, seed):
 
 
 def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0,
-           inj_m=0, mag=100.0, seed=0, split=0, pf=0):
-    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 1, split, pf))
+           inj_m=0, mag=100.0, seed=0, split=0, pf=0, ft=1):
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, ft, split, pf))
     N = 1 << logNi
     bs = ntiles * BS
     x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
@@ -135,3 +135,112 @@ def test_table_in_registers_or_read_per_tile():
         assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("double2", logNi)
         sp, x, y, c, fl = run_ft("double2", logNi, BS, n, ntiles, tbs, gap, inj_mode=0, correct=1)
         assert c[1] == 0 and not fl
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("logNi,BS,n,split", [(8, 4, 16, 0), (7, 8, 8, 0), (10, 1, 8, 1), (6, 8, 4, 0)])
+def test_delayed_batch_correction_flavour(dtype, logNi, BS, n, split):
+    # the `_fd` kernels keep per-thread sums of the group's inputs and outputs and patch the
+    # located tile with FFT(sum x) - sum y instead of recomputing it from its input
+    ntiles, tbs, gap = 22, 4, 3                    # ragged last group
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=1, correct=1, split=split, ft=2)
+    groups = O.tile_groups(ntiles, tbs, gap)
+    injs = O.reference_injections(groups, tbs, 100.0)
+    assert c[0] == len(groups)
+    assert c[1] == len(injs) == c[2] and c[3] == 0
+    assert sorted(t for _, t in fl) == sorted(i.tile for i in injs)
+    ref = O.fft_ref(x)
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)
+    # tile by tile against the oracle's delayed correction of the same group
+    xt = x.reshape(ntiles, BS, -1)
+    yt = O.fft_ref(xt)
+    ct = simlib.ctype_of(dtype)
+    for inj in injs:
+        g = next(gr for gr in groups if inj.tile in gr)
+        yg = yt[g].astype(ct)
+        yg[g.index(inj.tile), inj.s, :] += inj.mag
+        want = O.delayed_batch_correction(xt[g], yg, g.index(inj.tile), n, dtype)
+        got = y.reshape(ntiles, BS, -1)[inj.tile]
+        assert O.rel_l2(got, want) < O.tolerance(dtype, logNi)
+    # without correction the error stays, and a clean run is untouched by the extra sums
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=0, correct=1, split=split, ft=2)
+    assert c[1] == 0 and O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+
+
+def test_delayed_batch_correction_ragged_rows():
+    # a last tile with fewer transforms than BS: the patch reads and writes only rows that exist
+    dtype, logNi, BS, n = "double2", 7, 8, 8
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 2))
+    N, bs = 1 << logNi, 8 * 5 + 3
+    ntiles = (bs + BS - 1) // BS
+    x = rnd((bs, N), 9).astype(np.complex128)
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = ntiles, bs, 3, 2
+    counters = np.zeros(8, dtype=np.uint64)
+    flagged = np.full(2 * 64, -7, dtype=np.int64)
+    ka.ft.counters, ka.ft.flagged, ka.ft.flagged_cap = counters.ctypes.data, flagged.ctypes.data, 64
+    ka.ft.correct, ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_mag = 1, 2, 1 << 30, ntiles - 1, 100.0
+    ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
+    cv = O.dft_checksum_vector(N, dtype).astype(np.complex128)
+    ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
+    y = simlib.run_sim(sp, x, bs * N, ka, (ntiles + 2) // 3, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
+    assert counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == ntiles - 1
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+
+
+def _ft_args(ka, ntiles, correct, inj_tile, mag, cap=64):
+    counters = np.zeros(8, dtype=np.uint64)
+    flagged = np.full(2 * cap, -7, dtype=np.int64)
+    ka.ft.counters, ka.ft.flagged, ka.ft.flagged_cap = counters.ctypes.data, flagged.ctypes.data, cap
+    ka.ft.correct, ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_mag = correct, 2, 1 << 30, inj_tile, mag
+    ka.ft.inj_s, ka.ft.inj_m = 1, 0
+    ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
+    return counters, flagged
+
+
+@pytest.mark.parametrize("ft", [1, 2])
+@pytest.mark.parametrize("dtype,logNi,BS,n,log_ncols", [("double2", 7, 16, 8, 8), ("float2", 8, 16, 16, 6)])
+def test_column_kernel_corrects_an_injected_tile(ft, dtype, logNi, BS, n, log_ncols):
+    # recompute (ft=1) and delayed batch correction (ft=2) in a column launch: the patch of
+    # the delayed flavour is formed before the inter-launch twiddle and multiplied by it
+    sp = KernelSpec(KernelKey(dtype, "col", logNi, BS, n, ft))
+    Ni, ncols, outer = 1 << logNi, 1 << log_ncols, 3
+    x = rnd((outer, Ni, ncols), 5)
+    ka = simlib.KArgs()
+    ka.ntiles = outer * ncols // BS
+    ka.thread_bs, ka.tb_gap, ka.log_ncols = 3, 2, log_ncols
+    lo_bits, hi, lo = simlib.split_tables(logNi + log_ncols, dtype)
+    ka.tw_lo_bits = lo_bits
+    counters, flagged = _ft_args(ka, ka.ntiles, 1, 7, 1e4)
+    cv = O.dft_checksum_vector(Ni, dtype).astype(np.complex128)
+    ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
+    grid = (ka.ntiles + 2) // 3
+    y = simlib.run_sim(sp, x, x.size, ka, grid, simlib.twiddle_table(Ni, dtype), hi, lo, ck=ck).reshape(outer, Ni, ncols)
+    assert counters[0] == grid and counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == 7
+    ref = np.fft.fft(x.astype(simlib.ctype_of(dtype)).astype(np.complex128), axis=1)
+    k = np.arange(Ni)[:, None]
+    col = np.arange(ncols)[None, :]
+    ref = ref * np.exp(-2j * np.pi * ((k * col) % (Ni * ncols)) / (Ni * ncols))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)
+
+
+@pytest.mark.parametrize("ft", [1, 2])
+@pytest.mark.parametrize("dtype,logA,BS,n,logQ,logC", [("double2", 8, 8, 8, 0, 4), ("float2", 8, 16, 16, 3, 4)])
+def test_transposing_kernel_corrects_an_injected_tile(ft, dtype, logA, BS, n, logQ, logC):
+    sp = KernelSpec(KernelKey(dtype, "rowT", logA, BS, n, ft))
+    A, Q, Cc = 1 << logA, 1 << logQ, 1 << logC
+    bs = 2
+    x = rnd((bs, Cc, Q, A), 7)
+    ka = simlib.KArgs()
+    ka.ntiles = bs * Q * Cc // BS
+    ka.thread_bs, ka.tb_gap = 2, 3
+    ka.logQ, ka.logC, ka.logN = logQ, logC, logA + logQ + logC
+    counters, flagged = _ft_args(ka, ka.ntiles, 1, ka.ntiles - 1, 1e4)
+    cv = O.dft_checksum_vector(A, dtype).astype(np.complex128)
+    ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
+    grid = (ka.ntiles + 1) // 2
+    y = simlib.run_sim(sp, x, x.size, ka, grid, simlib.twiddle_table(A, dtype), ck=ck).reshape(bs, A, Q, Cc)
+    assert counters[0] == grid and counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == ka.ntiles - 1
+    xc = x.astype(simlib.ctype_of(dtype)).astype(np.complex128)
+    ref = np.transpose(np.fft.fft(xc, axis=3), (0, 3, 2, 1))
+    assert O.rel_l2(y, ref) < O.tolerance(dtype, logA)

@@ -96,6 +96,144 @@ def test_reference_cadence_matches_oracle_model(dt, logN, bs, tbs):
     assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
 
 
+@pytest.mark.parametrize("dt,logN,bs", [("float2", 10, 64), ("double2", 10, 16), ("float2", 13, 32), ("double2", 13, 8)])
+def test_reference_checksum_table_clean_run(dt, logN, bs):
+    # the table the reference's kernels actually read (abft.h:21-61: angles rounded to float
+    # before the division): decisions on clean data must equal the oracle model fed the same
+    # table.  At 8192 points that table is off by up to 3e-3 rad; the model says whether the
+    # residual this leaves on clean data stays below the rule, the GPU has to agree.
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=4)
+    plan.set_checksum_mode("reference")
+    plan.set_tb_gap(0, 5)
+    x = make(bs, 1 << logN, dt, 40 + logN)
+    y, c = run(plan, x)
+    row = O.PlanRow.from_list(plan.plan_row())
+    dec, _ = O.ft_plan_model(x, row, dt, 4, [5], None, table_mode="reference")
+    exact, _ = O.ft_plan_model(x, row, dt, 4, [5], None, table_mode="exact")
+    worst = max(abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3 for d in dec[0])
+    worst_exact = max(abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3 for d in exact[0])
+    print(f"clean-data ratio to the threshold: reference table {worst:.3e}, exact table {worst_exact:.3e}", flush=True)
+    assert all(r < 0.67 or r > 1.5 for r in (abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3 for d in dec[0]))
+    model = sorted((0, d.tile) for d in dec[0] if d.detected)
+    assert sorted(c["flagged"]) == model and c["detected"] == len(model)
+    assert c["checked"] == plan.grid(0, bs)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)       # a false alarm only recomputes
+    plan.close()
+
+
+@pytest.mark.parametrize("dt,bs", [("float2", 64), ("double2", 16)])
+@pytest.mark.parametrize("tbs", [2, 4])
+def test_reference_checksum_table_reference_cadence(dt, bs, tbs):
+    # if_err=1 at 2^10 with the reference's own table: every block injects 100 into element 0
+    # of one of its tiles, detects, locates and recomputes it; decisions against the model run
+    # with table_mode="reference"
+    logN = 10
+    plan = turbofft_amd.TurboFFT(logN, dt, if_err=1, thread_bs=tbs)
+    plan.set_checksum_mode("reference")
+    plan.set_tb_gap(0, 7)
+    x = make(bs, 1 << logN, dt, 77)
+    y, c = run(plan, x)
+    row = O.PlanRow.from_list(plan.plan_row())
+    groups = O.tile_groups(O.launch_geometry(row, bs)[0].ntiles, tbs, 7)
+    injs = O.reference_injections(groups, tbs, 100.0)
+    dec, _ = O.ft_plan_model(x, row, dt, tbs, [7], injs, table_mode="reference")
+    for d in dec[0]:
+        ratio = abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3
+        assert ratio < 0.67 or ratio > 1.5, "test case sits on the detection threshold"
+    model = sorted((0, d.tile) for d in dec[0] if d.detected)
+    assert model == sorted((0, i.tile) for i in injs)
+    assert sorted(c["flagged"]) == model and c["detected"] == len(injs) == c["corrected"]
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    assert c0["detected"] == 0 and np.array_equal(y, y0)
+    # back to the exact table: same decisions on this case, same corrected output
+    plan.set_checksum_mode("exact")
+    plan.set_injection(1, mag=100.0)
+    y1, c1 = run(plan, x)
+    assert sorted(c1["flagged"]) == model and np.array_equal(y1, y0)
+    plan.close()
+
+
+@pytest.mark.parametrize("dt,logN,bs", CASES)
+@pytest.mark.parametrize("tbs", [2, 8])
+def test_delayed_batch_correction_matches_oracle_model(dt, logN, bs, tbs):
+    # correct=2: the located tile is patched with FFT(sum x) - sum y of its group instead of
+    # being recomputed from its input (fft_codegen.py:355-357,421-423 live sums, :401-404,
+    # 427-429 and test.ipynb cell 0 for the patch).  Same detections as the recompute flavour;
+    # the patched result meets the accuracy bar (to rounding, not bit for bit) and every
+    # patched tile agrees with the oracle's delayed_batch_correction of the same group.
+    plan = turbofft_amd.TurboFFT(logN, dt, if_err=1, thread_bs=tbs)
+    plan.set_ft_params(1000.0, 1e-3, correct=2)
+    gaps = [7, 5, 3][:plan.launches]
+    for i, g in enumerate(gaps):
+        plan.set_tb_gap(i, g)
+    x = make(bs, 1 << logN, dt, logN + 1)
+    row = O.PlanRow.from_list(plan.plan_row())
+    if logN <= 10:
+        mag = 100.0
+    else:
+        clean, _ = O.ft_plan_model(x, row, dt, tbs, gaps, None)
+        mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[-1])) / 0.366))
+    plan.set_injection(1, mag=mag)
+    y, c = run(plan, x)
+    geoms = O.launch_geometry(row, bs)
+    last = geoms[-1]
+    groups = O.tile_groups(last.ntiles, tbs, gaps[plan.launches - 1])
+    injs = O.reference_injections(groups, tbs, mag)
+    dec, _ = O.ft_plan_model(x, row, dt, tbs, gaps, injs)
+    for dl in dec:
+        for d in dl:
+            ratio = abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3
+            assert ratio < 0.67 or ratio > 1.5, "test case sits on the detection threshold"
+    model = sorted((li, d.tile) for li, dl in enumerate(dec) for d in dl if d.detected)
+    assert model == sorted((plan.launches - 1, i.tile) for i in injs)
+    assert sorted(c["flagged"]) == model
+    assert c["detected"] == len(injs) == c["corrected"] and c["uncorrectable"] == 0
+    ref = O.fft_ref(x)
+    assert O.rel_l2(y, ref) <= O.tolerance(dt, logN)
+    worst = max(O.rel_l2(y[b], ref[b]) for b in range(bs))
+    assert worst <= O.tolerance(dt, logN) * 2
+    # the patch against the oracle's, tile by tile, for the single-launch plans (the tiles of a
+    # last launch are rows of the previous launch's output, compared through the bar above)
+    if plan.launches == 1:
+        BS, n = plan.BS[0], plan.n[0]
+        xt = last.gather(x)
+        yt = O.fft_ref(xt).astype(cdtype(dt))
+        got = last.gather(y)
+        for inj in injs[:16]:
+            g = next(gr for gr in groups if inj.tile in gr)
+            yg = yt[g].copy()
+            yg[g.index(inj.tile), inj.s, :] += inj.mag
+            want = O.delayed_batch_correction(xt[g], yg, g.index(inj.tile), n, dt)
+            assert O.rel_l2(got[inj.tile], want) <= O.tolerance(dt, logN)
+    # without injection the flavour is transparent
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    assert c0["detected"] == 0 and O.rel_l2(y0, ref) <= O.tolerance(dt, logN)
+    plan.close()
+
+
+def test_delayed_batch_correction_host_chosen_tiles_and_earlier_launch():
+    plan = turbofft_amd.TurboFFT(15, "double2", if_ft=1, thread_bs=2)
+    plan.set_ft_params(1000.0, 1e-3, correct=2)
+    plan.set_injection(2, launch=0, every=1 << 30, tile_phase=9, s=3, m=1, mag=1000.0)
+    x = make(4, 1 << 15, "double2", 5)
+    y, c = run(plan, x)
+    assert c["flagged"] == [(0, 9)] and c["corrected"] == 1
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance("double2", 15)
+    plan.close()
+    # ragged single-launch batch: the last tile holds fewer transforms than BS
+    plan = turbofft_amd.TurboFFT(7, "float2", if_ft=1, thread_bs=3)
+    plan.set_ft_params(1000.0, 1e-3, correct=2)
+    bs = plan.BS[0] * 10 + 3
+    plan.set_injection(2, every=1 << 30, tile_phase=10, s=1, m=0, mag=1000.0)
+    x = make(bs, 128, "float2", 6)
+    y, c = run(plan, x)
+    assert c["flagged"] == [(0, 10)] and c["corrected"] == 1
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance("float2", 7)
+    plan.close()
+
+
 def test_reference_default_magnitude_is_below_the_rule_at_8192_points():
     # the model of the reference rule predicts NO detection for err_inj=100 on a
     # U[-1,1) fp32 8192-point tile (|delta| = 36.6, mag ~ 1.5e5): the GPU must agree

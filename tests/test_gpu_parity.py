@@ -474,6 +474,90 @@ def test_cli_bench_modes():
             assert int(f[1]) + int(f[2]) == 22 and float(f[3]) > 0 and float(f[4]) > 0 and float(f[5]) > 0
 
 
+@pytest.mark.parametrize("extra", [[], ["--if_ft", "1", "--thread_bs", "4"], ["--if_ft", "1", "--if_err", "1", "--thread_bs", "2"]])
+def test_cli_all_batch_sizes_sweep(extra):
+    # --if_bench 1 (main.cu:114-128): for every logN all batch sizes 1, 2, 4 ... 2^(param_1 - logN),
+    # one metric line each, plain and fault tolerant
+    p1 = 14
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "1", "--datatype", "1", "--param_1", str(p1),
+                        "--logN_begin", "9", "--logN_end", "11"] + extra, capture_output=True, text=True, timeout=300)
+    print(r.stdout[-3000:], r.stderr[-500:], flush=True)
+    assert r.returncode == 0
+    lines = [[v.strip() for v in ln.split(",")] for ln in r.stdout.splitlines() if ln.startswith("turboFFT, ")]
+    want = [(logN, lb) for logN in (9, 10, 11) for lb in range(0, p1 - logN + 1)]
+    assert [(int(f[1]), int(f[2])) for f in lines] == want          # batch column doubles from 1 up to the cap
+    for f in lines:
+        ms, gflops, gbs = float(f[3]), float(f[4]), float(f[5])
+        N, bs = 1 << int(f[1]), 1 << int(f[2])
+        assert ms > 0
+        # the metric columns are the reference's formulas of the time column (main.cu:68-69),
+        # which is printed with three decimals
+        lo, hi = max(ms - 6e-4, 1e-7), ms + 6e-4
+        assert 5.0 * N * int(f[1]) * bs / hi / 1e6 - 2e-3 <= gflops <= 5.0 * N * int(f[1]) * bs / lo / 1e6 + 2e-3
+        assert 2.0 * N * bs * 16 / hi / 1e6 - 2e-3 <= gbs <= 2.0 * N * bs * 16 / lo / 1e6 + 2e-3
+    ft = [ln for ln in r.stdout.splitlines() if ln.startswith("turboFFT_ft, ")]
+    assert len(ft) == (len(want) if extra else 0)
+    if "--if_err" not in extra:
+        assert all("detected=0," in ln for ln in ft)
+
+
+def test_cli_gpu_flag_selects_the_plan_table(tmp_path):
+    # CommandLineParser.h:93-109: --gpu <name> reads param/<name>/param_<T>.csv and T4 lowers the
+    # sweep to logBS + logN = 26; a name without tables is reported, not ignored
+    pdir = os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param")
+    name = "unit_test_gpu_%d" % os.getpid()
+    os.makedirs(os.path.join(pdir, name))
+    try:
+        src = os.path.join(pdir, "gfx950", "reference_shapes_double2.csv")
+        with open(src) as f, open(os.path.join(pdir, name, "param_double2.csv"), "w") as g:
+            g.write(f.read())
+        common = ["--if_bench", "0", "--if_verify", "1", "--logN", "15", "--bs", "2", "--bs_end", "2", "--datatype", "1"]
+        r = subprocess.run([turbofft_amd.CLI_PATH] + common + ["--gpu", name], capture_output=True, text=True, timeout=120)
+        print(r.stdout[-1500:], r.stderr[-300:], flush=True)
+        assert r.returncode == 0 and f"param/{name}/param_double2.csv" in r.stdout
+        assert "Compare finished." in r.stdout and "Error detected" not in r.stdout
+        r = subprocess.run([turbofft_amd.CLI_PATH] + common + ["--gpu", "no_such_gpu"], capture_output=True, text=True, timeout=120)
+        assert r.returncode != 0 and "Failed to open file." in r.stdout
+        r = subprocess.run([turbofft_amd.CLI_PATH] + common + ["--gpu", "MI355X"], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0 and "<built-in gfx950>" in r.stdout
+    finally:
+        import shutil
+        shutil.rmtree(os.path.join(pdir, name))
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "2", "--gpu", "T4", "--param", os.path.join(pdir, "gfx950", "param_float2.csv"),
+                        "--logN_begin", "12", "--logN_end", "12"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "param_1: 26" in r.stdout and "turboFFT, 12, 14," in r.stdout
+
+
+def test_cli_sync_timing_line():
+    # --if_sync 1 adds the figure the reference's loop measures (a host wait after every launch,
+    # main.cu:53-62) beside the default one; it can only be slower
+    r = subprocess.run([turbofft_amd.CLI_PATH, "--if_bench", "2", "--datatype", "0", "--param_1", "24", "--if_sync", "1",
+                        "--logN_begin", "16", "--logN_end", "17"], capture_output=True, text=True, timeout=120)
+    print(r.stdout[-1500:], r.stderr[-300:], flush=True)
+    assert r.returncode == 0
+    a = [float(ln.split(",")[3]) for ln in r.stdout.splitlines() if ln.startswith("turboFFT, ")]
+    b = [float(ln.split(",")[3]) for ln in r.stdout.splitlines() if ln.startswith("turboFFT_sync, ")]
+    assert len(a) == len(b) == 2 and all(y > 0.9 * x for x, y in zip(a, b))
+
+
+def test_overlapping_buffers_are_rejected():
+    torch = _torch()
+    for logN, dt in ((10, "float2"), (16, "float2")):
+        plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1)
+        N, bs = 1 << logN, 4
+        buf = torch.zeros(4 * N * bs, dtype=torch.complex64, device="cuda")
+        st = torch.cuda.current_stream().cuda_stream
+        for in_off, out_off in ((0, 0), (0, N * bs // 2), (N * bs // 2, 0)):
+            with pytest.raises(turbofft_amd.TurboFFTError, match="overlaps"):
+                plan.exec(buf.data_ptr() + 8 * in_off, buf.data_ptr() + 8 * out_off, bs, st)
+        if plan.launches > 1:                  # `in` inside the workspace half of `out`
+            with pytest.raises(turbofft_amd.TurboFFTError, match="overlaps"):
+                plan.exec(buf.data_ptr() + 8 * N * bs, buf.data_ptr(), bs, st)
+        plan.exec(buf.data_ptr() + 8 * plan.out_elems(bs), buf.data_ptr(), bs, st)      # adjacent is fine
+        torch.cuda.synchronize()
+        plan.close()
+
+
 VARIANTS_DIR = os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param", "gfx950")
 
 
@@ -563,3 +647,9 @@ def test_exec_inside_a_hip_graph(dt, logN, bs, ft):
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay {rep} differs from the eager run"
         assert O.rel_l2(got.cpu().numpy(), O.fft_ref(x.cpu().numpy())) <= O.tolerance(dt, logN)
+    if ft:
+        # the groups-checked counter lives on the device: replays count like eager executions
+        # (1 warm-up + 3 replays + 3 eager runs; the capture itself executes nothing)
+        c = plan.ft_counters()
+        assert c["checked"] == 7 * sum(plan.grid(i, bs) for i in range(plan.launches)) and c["detected"] == 0
+    plan.close()

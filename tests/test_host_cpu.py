@@ -125,13 +125,22 @@ def test_checksum_vector_exact_matches_oracle(dtype, N):
 
 
 @pytest.mark.parametrize("dtype", ["float2", "double2"])
-def test_checksum_vector_reference_mode_matches_oracle(dtype):
-    # same float-rounded-angle arithmetic on both sides; libm vs numpy sin/cos may
-    # differ in the last ulp of float, so compare to a few ulps of the magnitude
-    N = 256
+@pytest.mark.parametrize("N", [256, 1024])
+def test_checksum_vector_reference_mode_pinned_by_multiprecision(dtype, N):
+    # the library's mode 1 against abft.h:21-61 evaluated in multiprecision (tests/mp_checksum.py),
+    # not against the numpy restatement of the same lines
+    import mp_checksum as M
+    rows = [0, 1, 2, N // 3, N // 2, N - 1]
+    want = M.checksum_rows(N, rows)
     a = turbofft_amd.checksum_vector(N, dtype, "reference")
+    tol = 2e-5 if dtype == "float2" else 1e-12
+    assert max(abs(complex(a[i]) - want[i]) for i in rows) < tol
+    for v in ("unrounded_angle", "float_two_pi"):
+        bad = M.checksum_rows(N, rows, v)
+        assert max(abs(bad[i] - want[i]) for i in rows) > 5 * tol
+    # and bit-for-bit the oracle's table in fp64, where libm and numpy share cos/sin of a double
     b = O.dft_checksum_vector(N, dtype, "reference")
-    assert np.max(np.abs(a - b)) <= np.max(np.abs(b)) * (2e-5 if dtype == "float2" else 1e-6)
+    assert np.max(np.abs(a - b)) <= np.max(np.abs(b)) * (2e-5 if dtype == "float2" else 1e-13)
 
 
 def test_bad_arguments_are_reported_not_fatal():

@@ -82,10 +82,39 @@ def test_checksum_reference_mode_matches_exact_for_small_N():
         a = O.dft_checksum_vector(N, "double2", "reference")
         b = O.dft_checksum_vector(N, "double2", "exact")
         assert np.max(np.abs(a - b)) < 1e-5
-    # and visibly wrong for large N (the known quirk of the reference)
-    a = O.dft_checksum_vector(1024, "double2", "reference")
-    b = O.dft_checksum_vector(1024, "double2", "exact")
-    assert 1e-6 < np.max(np.abs(a - b)) / np.max(np.abs(b)) < 1e-1
+
+
+REF_ROWS = {256: [0, 1, 2, 85, 128, 255], 1024: [0, 1, 3, 341, 512, 1023], 8192: [1, 2731, 8191]}
+WRONG_READINGS = ["unrounded_angle", "float_two_pi", "r_shifted", "positive_angle", "exact_sqrt3"]
+
+
+@pytest.mark.parametrize("N", [256, 1024, 8192])
+def test_checksum_reference_mode_pinned_by_multiprecision(N):
+    """abft.h:21-61 evaluated independently: float32 angle from struct, cos/sin and the sum
+    over j in 40-digit arithmetic.  The fp64 variant of the oracle must agree to accumulation
+    rounding (~1e-15*sqrt(N)), the fp32 variant to the rounding of N float additions; every
+    wrong reading of the source lines (angle not rounded to float, 2*pi rounded first, r
+    started at the wrong residue, +i exponent, exact sqrt(3)/2 instead of the float literal,
+    and -- where i*j exceeds 2^24 -- the index product rounded first) is off by orders of
+    magnitude more and must be told apart."""
+    import mp_checksum as M
+    rows = REF_ROWS[N]
+    want = M.checksum_rows(N, rows)
+    o64 = O.dft_checksum_vector(N, "double2", "reference")
+    o32 = O.dft_checksum_vector(N, "float2", "reference")
+    tol64, tol32 = 4e-15 * N ** 0.5 * 4, 2e-5
+    assert max(abs(o64[i] - want[i]) for i in rows) < tol64
+    assert max(abs(complex(o32[i]) - want[i]) for i in rows) < tol32
+    wrong = WRONG_READINGS + (["float_index_product"] if N == 8192 else [])
+    for v in wrong:
+        bad = M.checksum_rows(N, rows, v)
+        d = max(abs(bad[i] - want[i]) for i in rows)
+        assert d > 100 * tol64, (v, d)
+        if v != "exact_sqrt3":            # 1.5e-8 per term: below the fp32 accumulation noise
+            assert d > 5 * tol32, (v, d)
+    # the known quirk of the reference table: visibly wrong against the exact vector
+    b = O.dft_checksum_vector(N, "double2", "exact")
+    assert 1e-6 < np.max(np.abs(o64 - b)) / np.max(np.abs(b)) < 1e-1
 
 
 def test_checksum_table_offsets():
@@ -294,3 +323,34 @@ def test_rule_saturates_for_long_subffts():
             seen[(Ni, mag)] = d.detected
         assert abs(ratios[0] / ratios[1] - 1) < 1e-3          # saturated: independent of the magnitude
     assert seen[(256, 1e12)] and not seen[(2048, 1e12)]
+
+
+# ---------------- delayed batch correction ----------------------------------
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("Ni,n,BS,T", [(64, 8, 4, 4), (256, 16, 2, 8), (1024, 8, 1, 3)])
+def test_delayed_batch_correction_restores_the_clean_transform(dtype, Ni, n, BS, T):
+    # linearity pins it: whatever the error on tile k looks like (one output, a whole
+    # sub-FFT shifted as after an input-side upset, dense noise), y_k + FFT(sum x) - sum y is
+    # the clean transform of x_k.  A flipped sign doubles the error, a dropped sum leaves
+    # garbage of the size of the data, a wrong k patches a clean tile: all fail the bar.
+    x = rng_cplx((T, BS, Ni), Ni + T)
+    clean = O.fft_ref(x)
+    tol = O.tolerance(dtype, int(math.log2(Ni))) * math.sqrt(T) * 2
+    rng = np.random.default_rng(5)
+    for k in range(T):
+        for shape in ("one", "row", "dense"):
+            y = clean.copy()
+            if shape == "one":
+                y[k, BS - 1, 3] += 100.0
+            elif shape == "row":
+                y[k, 0, :] += 100.0                     # x[k,0,0] += 100 after the input checksum
+            else:
+                y[k] += rng.standard_normal((BS, Ni)) * 50
+            fixed = O.delayed_batch_correction(x, y, k, n, dtype)
+            assert O.rel_l2(fixed, clean[k]) < tol, (k, shape)
+            assert O.rel_l2(y[k], clean[k]) > 100 * tol
+    # the patch goes to the located tile only: patching another tile moves the error there
+    y = clean.copy()
+    y[1, 0, :] += 100.0
+    wrong = O.delayed_batch_correction(x, y, 0, n, dtype)
+    assert O.rel_l2(wrong, clean[0]) > 100 * tol

@@ -62,6 +62,8 @@ def lib() -> C.CDLL:
     L.turbofft_exec_inverse.argtypes = [vp, vp, vp, ll, vp]
     L.turbofft_exec_host.argtypes = [vp, vp, vp, ll]
     L.turbofft_time.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_time_sync.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_set_checksum_mode.argtypes = [vp, i]
     L.turbofft_time_launches.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_plan_info.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i), C.POINTER(i),
                                      C.POINTER(C.c_size_t), C.POINTER(i)]
@@ -275,6 +277,12 @@ class TurboFFT:
         _check(lib().turbofft_time(self._h, in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
         return ms.value
 
+    def time_sync(self, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0) -> float:
+        """The reference's timing protocol: the host waits after every launch (main.cu:53-62)."""
+        ms = C.c_float()
+        _check(lib().turbofft_time_sync(self._h, in_ptr, out_ptr, bs, warmup, reps, stream, C.byref(ms)))
+        return ms.value
+
     def time_launches(self, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0):
         """Mean duration of every launch of the plan (HIP events around each launch)."""
         ms = (C.c_float * 3)()
@@ -282,8 +290,13 @@ class TurboFFT:
         return list(ms)[: self.launches]
 
     # ---- fault tolerance ----
-    def set_ft_params(self, err_smoothing: float = 1000.0, err_threshold: float = 1e-3, correct: bool = True):
+    def set_ft_params(self, err_smoothing: float = 1000.0, err_threshold: float = 1e-3, correct=True):
+        """correct: 0/False detect only, 1/True recompute the located tile, 2 delayed batch correction."""
         _check(lib().turbofft_set_ft_params(self._h, err_smoothing, err_threshold, int(correct)))
+
+    def set_checksum_mode(self, mode: str):
+        """"exact" (default) or "reference": the reference's float-rounded-angle table (abft.h:21-61)."""
+        _check(lib().turbofft_set_checksum_mode(self._h, {"exact": 0, "reference": 1}[mode]))
 
     def set_injection(self, mode: int, launch: int = -1, every: int = 1, tile_phase: int = 0, s: int = 0, m: int = 0,
                       mag: float = 100.0):
@@ -299,7 +312,7 @@ class TurboFFT:
         _check(lib().turbofft_get_ft_counters(self._h, *[C.byref(t) for t in v], fl, cap, C.byref(n)))
         flagged = [(fl[2 * i], fl[2 * i + 1]) for i in range(n.value)]
         return {"checked": v[0].value, "detected": v[1].value, "corrected": v[2].value,
-                "uncorrectable": v[3].value, "flagged": flagged}
+                "uncorrectable": v[3].value, "flagged": flagged, "flagged_truncated": v[1].value > n.value}
 
     # ---- metrics (main.cu:68-69) ----
     def gflops(self, bs: int, ms: float) -> float:

@@ -92,6 +92,7 @@ class KernelSpec:
         self.n = k.n
         self.kind = k.kind
         self.ft = bool(k.ft)
+        self.dc = int(k.ft) == 2    # delayed batch correction: sums of the group's inputs and outputs per thread
         self.split = bool(k.split)
         self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
         self.xl = bool(k.xl)        # last (radix 2/4/8) pass across lanes instead of through LDS
@@ -101,6 +102,8 @@ class KernelSpec:
         self.Tr = self.Ni // self.n              # threads per sub-FFT
         self.threads = self.Tr * self.BS
         self.E = self.Ni * self.BS
+        if self.dc and self.pf:
+            raise ValueError(f"{k}: delayed batch correction has no prefetching flavour")
         if self.threads % WAVE or self.threads > 1024:
             raise ValueError(f"{k}: {self.threads} threads per block (need a multiple of 64, <= 1024)")
         # thread map per pass: 'major' (s = tx / Tr) or 'minor' (s = tx % BS)
@@ -187,6 +190,7 @@ class KernelEmitter:
         # transposing kernels measured 1-9 % slower that way and keep plain global pointers.
         buf = spec.kind == "row1"
         self.GLD, self.GST = ("GLDU", "GSTU") if buf else ("GLDG", "GSTG")
+        self.GLDC = self.GLD            # cached load of the same form (re-reads of a tile just stored)
         # Non-temporal variants for the tile data only (it is touched once); twiddles and the
         # checksum table are re-read by every tile and stay on the cached path.
         nt = int(spec.key.nt)
@@ -488,6 +492,8 @@ class KernelEmitter:
             if sp.BS > 1:
                 c("if ((row0 + s) < a.nrows) {")
                 c.ind += 1
+            if sp.dc:
+                self.emit_patch_load(c, [f"{self.GLDC}(out, ubase, {sp.Tr * e}, go)" for e in range(sp.n)])
             if self.pair_access():
                 c("if (((unsigned long long)out & 15ull) == 0ull) {")
                 c.ind += 1
@@ -508,12 +514,31 @@ class KernelEmitter:
             c("const unsigned col = (ct << %d) + s;" % ilog2(sp.BS))
             self.emit_interlaunch_twiddle(c)
             c("const unsigned go = s + (x << a.log_ncols);")
+            if sp.dc:
+                self.emit_patch_load(c, [f"{self.GLDC}(out, ubase, {e} * gstep, go)" for e in range(sp.n)])
             for e in range(sp.n):
                 c(f"{self.GST}(out, ubase, {e} * gstep, go, r[{self.out_reg(e)}]);")
         else:
             c("const unsigned go = s + (x << ls);")
+            if sp.dc:
+                self.emit_patch_load(c, [f"{self.GLDC}(out, ubase_out, {e} * gstep, go)" for e in range(sp.n)])
             for e in range(sp.n):
                 c(f"{self.GST}(out, ubase_out, {e} * gstep, go, r[{self.out_reg(e)}]);")
+
+    def emit_patch_load(self, c: Code, loads: Sequence[str]):
+        """Extra trip of a delayed-correction kernel: the registers hold the correction term
+        of the located tile; add what the tile's earlier trip stored, so that the stores that
+        follow write the patched result."""
+        sp = self.s
+        c("if (is_redo) {")
+        c.ind += 1
+        c(f"{self.T2} pv[{sp.n}];")
+        for e, ld in enumerate(loads):
+            c(f"pv[{e}] = {ld};")
+        for e in range(sp.n):
+            c(f"r[{self.out_reg(e)}] = cadd(r[{self.out_reg(e)}], pv[{e}]);")
+        c.ind -= 1
+        c("}")
 
     def emit_interlaunch_twiddle(self, c: Code):
         """r[k] *= W_(Ni*ncols)^(col*k), k = x + Tr*e: base and step come from the
@@ -600,6 +625,10 @@ class KernelEmitter:
                 c("SCHED_FENCE();")
         c("acc += acy;")
         c("fin1 += acc; fin2 += cntf * acc;")
+        if sp.dc:
+            # per-thread sum of the group's inputs (fft_codegen.py:355-357), taken before the injection
+            for e in range(sp.n):
+                c(f"sx[{e}] = cadd(sx[{e}], r[{e}]);")
         # the injected element is one of the first Ni/n of its sub-FFT (register 0 of thread
         # x = m; the reference injects at m = 0)
         c(f"r[0].x += (inj_hit && s == (unsigned)a.ft.inj_s && x == (unsigned)a.ft.inj_m) ? ({self.R})a.ft.inj_mag : ({self.R})0;")
@@ -628,8 +657,23 @@ class KernelEmitter:
             c(f"acc += r[{reg}].x * rp{ce}; acy += r[{reg}].y * rq{ce};")
         c("acc += acy;")
         c("fo1 -= acc; fo2 -= cntf * acc;")
+        if sp.dc:
+            # per-thread sum of the group's outputs as computed, before the inter-launch twiddle
+            # (fft_codegen.py:421-423)
+            for e in range(sp.n):
+                c(f"sy[{e}] = cadd(sy[{e}], r[{self.out_reg(e)}]);")
         c.ind -= 1
         c("}")
+        if sp.dc:
+            # extra trip: the registers hold FFT(sum of the group's inputs); what the located tile's
+            # stored result lacks is that minus the sum of the group's outputs (fft_codegen.py:401-404,
+            # 427-429; the notebook's b_out += FFT(A e) - B_out e with unit weights)
+            c("else {")
+            c.ind += 1
+            for e in range(sp.n):
+                c(f"r[{self.out_reg(e)}] = csub(r[{self.out_reg(e)}], sy[{e}]);")
+            c.ind -= 1
+            c("}")
 
     # ---------- phases ----------
     def emit_xlane_pass(self, c: Code, q: int) -> List[str]:
@@ -732,7 +776,18 @@ class KernelEmitter:
                     prio = bool(int(sp.key.nt) & 4)
                     if prio:
                         c("TFFT_WAVE_PRIO(3);")
+                    if sp.dc:
+                        c("if (!is_redo) {")
+                        c.ind += 1
                     self.emit_load(c)
+                    if sp.dc:
+                        c.ind -= 1
+                        c("} else {")
+                        c.ind += 1
+                        for e in range(sp.n):
+                            c(f"r[{e}] = sx[{e}];")
+                        c.ind -= 1
+                        c("}")
                     if prio:
                         c("TFFT_WAVE_PRIO(0);")
                     if sp.ft:
@@ -791,7 +846,7 @@ class KernelEmitter:
         c = Code()
         T2, R = self.T2, self.R
         c(f"// {sp.name}: {sp.kind} kernel, {T2}, Ni={sp.Ni}, BS={sp.BS}, n={sp.n}, passes={'x'.join(map(str, sp.passes))},")
-        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}{', cross-lane last pass' if sp.xl else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' if sp.ft else ''}")
+        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}{', cross-lane last pass' if sp.xl else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' + (' (delayed batch correction)' if sp.dc else '') if sp.ft else ''}")
         if sim:
             c(f'extern "C" void {sp.name}_sim(const {T2}* in, {T2}* out, const {T2}* tw, const tfft_kargs* ap, long long grid, const long long* limits)')
             c("{")
@@ -801,7 +856,7 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx;")
@@ -827,6 +882,9 @@ class KernelEmitter:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
                 if self.ft_table_resident():
                     c(f"{T2} cvr[{sp.n}];")
+                if sp.dc:
+                    c(f"{T2} sx[{sp.n}], sy[{sp.n}];")
+                    c(f"for (int e = 0; e < {sp.n}; ++e) {{ sx[e] = czero(sx[e]); sy[e] = czero(sy[e]); }}")
         # XCD-aware renumbering: hardware deals blocks round-robin to the 8 XCDs, so block
         # b runs on XCD b % 8.  Give every XCD chunks of `xcd_chunk` consecutive tiles (its
         # L2 then streams contiguous memory) while the 8 XCDs stay in one neighbourhood.
@@ -859,6 +917,11 @@ class KernelEmitter:
             c.ind -= 1
             c("}")
         if sp.ft:
+            # checksum groups run: one per block, counted once per launch by its first block
+            if sim:
+                c("if (pbx == 0) a.ft.counters[0] += (unsigned long long)grid;")
+            else:
+                c("if (blockIdx.x == 0 && tx == 0) atomicAdd(&a.ft.counters[0], (unsigned long long)grid);")
             c("long long redo_tile = -1; int extra = 0;")
             if self.ft_table_resident():
                 self.emit_ft_table_resident_load(c, sim)
@@ -917,8 +980,8 @@ class KernelEmitter:
         if sim:
             c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
             c.ind += 1
-            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
-            c("(void)r; (void)rn; (void)cvr; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
+            c("(void)r; (void)rn; (void)cvr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
         else:
             c("{")
             c.ind += 1

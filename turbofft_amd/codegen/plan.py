@@ -71,7 +71,9 @@ class KernelKey:
     logNi: int
     BS: int
     n: int
-    ft: int
+    ft: int          # 0 plain; 1 fused checksums, a located tile is recomputed from its input; 2 the same
+                     # checksums with delayed batch correction (per-thread sums of the group's inputs and
+                     # outputs, the located tile is patched with FFT(sum x) - sum y)
     split: int = 0   # 1: every LDS exchange moves re and im in two rounds through a half-size buffer
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
@@ -85,7 +87,7 @@ class KernelKey:
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ("_ft" if self.ft else ""))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:

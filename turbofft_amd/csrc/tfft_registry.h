@@ -10,7 +10,8 @@ typedef struct tfft_kernel_entry {
     const void* func;    // host-side kernel handle for hipLaunchKernel
     int datatype;        // 0 = float2, 1 = double2
     int kind;            // 0 = row1, 1 = col, 2 = rowT
-    int logNi, BS, n, ft;
+    int logNi, BS, n;
+    int ft;              // 0 plain, 1 fused checksums (recompute correction), 2 fused checksums with delayed batch correction
     int split;           // 1: re and im are exchanged through LDS in two rounds
     int pf;              // 1: the block prefetches its next tile (wants a persistent grid)
     int xl;              // 1: the last small-radix pass runs across lanes (DPP / ds_swizzle)

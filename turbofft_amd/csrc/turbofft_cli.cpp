@@ -14,12 +14,14 @@
 //   --if_bench 11/12                             the same two sweeps with hipFFT (cuFFT in the
 //                                                reference, main.cu:121)
 #include <hip/hip_runtime.h>
+#include <dlfcn.h>
 
 #include <cmath>
 #include <complex>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <iostream>
 #include <string>
 #include <vector>
@@ -35,10 +37,14 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
     bool if_ft = false, if_err = false;
     int datatype = 0, thread_bs = 1;
     int param_1 = 28, param_2 = 16;
+    bool param_1_given = false;
     int sm_cnt = 256, smem_size = 160;
     int logN_begin = 1, logN_end = 25;
     std::string gpu = "gfx950";
     std::string param_file_path;     // empty: built-in gfx950 table
+    bool param_given = false;        // --param names the CSV; otherwise --gpu selects it
+    bool if_sync = false;            // also print the reference's sync-after-every-launch timing
+    int ft_correction = 1;           // 1 recompute the located tile, 2 delayed batch correction
 
     static void displayHelp() {
         std::cout << "Usage: program [options]\n"
@@ -57,8 +63,10 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
                   << "  --if_err <0|1>       Enable (1) or disable (0) error injection.\n"
                   << "  --datatype <type>    0 for FP32, 1 for FP64.\n"
                   << "  --thread_bs <value>  Set batches per block to <value>.\n"
-                  << "  --gpu <str>          Set GPU spec.\n"
-                  << "  --param <file>       Plan CSV (default: built-in gfx950 table).\n"
+                  << "  --gpu <str>          Set GPU spec: selects param/<gpu>/param_<type>.csv (gfx950 and MI355X: the built-in table).\n"
+                  << "  --param <file>       Plan CSV (overrides the one --gpu selects).\n"
+                  << "  --if_sync <0|1>      Also time with a host wait after every launch, as the reference does.\n"
+                  << "  --ft_correction <1|2> With --if_err: recompute the located tile (1) or delayed batch correction (2).\n"
                   << "  --logN_begin/--logN_end <value>  Restrict the --if_bench sweep.\n"
                   << "  --param_1 <value>        logBS + logN of the --if_bench sweep (default 28; the reference derives it from --gpu).\n"
                   << "  -h, --help               Display this help message and exit.\n";
@@ -77,10 +85,12 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
         else if (!strcmp(name, "--datatype")) datatype = atoi(value);
         else if (!strcmp(name, "--thread_bs")) thread_bs = atoi(value);
         else if (!strcmp(name, "--gpu")) gpu = value;
-        else if (!strcmp(name, "--param")) param_file_path = value;
+        else if (!strcmp(name, "--param")) { param_file_path = value; param_given = true; }
+        else if (!strcmp(name, "--if_sync")) if_sync = atol(value);
+        else if (!strcmp(name, "--ft_correction")) ft_correction = atoi(value);
         else if (!strcmp(name, "--logN_begin")) logN_begin = atoi(value);
         else if (!strcmp(name, "--logN_end")) logN_end = atoi(value);
-        else if (!strcmp(name, "--param_1")) param_1 = atoi(value);
+        else if (!strcmp(name, "--param_1")) { param_1 = atoi(value); param_1_given = true; }
         else return false;
         return true;
     }
@@ -94,7 +104,29 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
                 std::cerr << "Invalid or incomplete argument: " << argv[i] << std::endl;
                 return EXIT_FAILURE + 1;
             }
+        resolveGpu();
         return 0;
+    }
+
+    // CommandLineParser.h:93-109: --gpu picks the plan CSV (../include/param/<gpu>/param_<T>.csv
+    // there) and the sweep constants (T4: logBS+logN = 26).  Here the tables live in
+    // param/<gpu>/ beside the library; "gfx950" (or "MI355X") is the table compiled into it.  The
+    // reference's own relative path is tried as well, so that its directory layout keeps working.
+    void resolveGpu() {
+        if (gpu == "T4") { if (!param_1_given) param_1 = 26; param_2 = 4; }
+        if (param_given || gpu == "gfx950" || gpu == "MI355X") return;
+        const std::string leaf = "/param/" + gpu + (datatype == 1 ? "/param_double2.csv" : "/param_float2.csv");
+        std::vector<std::string> tries;
+        Dl_info info;
+        if (dladdr((const void*)&turbofft_main, &info) && info.dli_fname) {
+            std::string lib = info.dli_fname;
+            size_t cut = lib.find_last_of('/');
+            tries.push_back((cut == std::string::npos ? std::string(".") : lib.substr(0, cut)) + leaf);
+        }
+        tries.push_back("../include" + leaf);
+        for (const std::string& t : tries)
+            if (std::ifstream(t).good()) { param_file_path = t; return; }
+        param_file_path = tries.front();       // reported as "Failed to open file." when the plan is made (readCSV.h:29-31)
     }
 
     void displayConfig() const {      // CommandLineParser.h:112-119
@@ -105,6 +137,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
         std::cout << "gpu: " << gpu << ", param_1: " << param_1 << ", param_2: " << param_2 << std::endl;
         std::cout << "sm_cnt: " << sm_cnt << "smem_size: " << smem_size << "param_file_path: "
                   << (param_file_path.empty() ? std::string("<built-in gfx950>") : param_file_path) << std::endl;
+        if (if_sync || ft_correction != 1) std::cout << "if_sync: " << if_sync << ", ft_correction: " << ft_correction << std::endl;
     }
 };
 
@@ -194,12 +227,22 @@ int test_turbofft(const ProgramConfig& cfg, int logN, long long bs, int ntest, B
     turbofft_plan_t* plan = turbofft_plan_create(logN, cfg.datatype, cfg.if_ft, cfg.if_err, cfg.thread_bs, csv);
     if (!plan) { printf("turboFFT, %d: %s\n", logN, turbofft_last_error()); return -1; }
     float ms = 0;
-    int rc = turbofft_time(plan, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms);
+    int rc = TURBOFFT_OK;
+    if (cfg.if_err && cfg.ft_correction == 2) rc = turbofft_set_ft_params(plan, 1000.0, 1e-3, 2);
+    if (!rc) rc = turbofft_time(plan, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms);
     if (rc) { printf("turboFFT, %d: %s\n", logN, turbofft_last_error()); turbofft_plan_destroy(plan); return rc; }
     double N = (double)(1ll << logN);
     double gflops = 5.0 * N * logN * (double)bs / ms * 1000.0 / 1e9;             // main.cu:68
     double gbs = N * (double)bs * (double)b.esize * 2.0 / ms * 1000.0 / 1e9;     // main.cu:69
     printf("turboFFT, %d, %d, %8.3f, %8.3f, %8.3f\n", logN, (int)log2((double)bs), ms, gflops, gbs);
+    if (cfg.if_sync) {
+        // the figure the reference's loop measures: the host waits after every launch (main.cu:53-62)
+        float ms_s = 0;
+        rc = turbofft_time_sync(plan, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms_s);
+        if (rc) { printf("turboFFT_sync, %d: %s\n", logN, turbofft_last_error()); turbofft_plan_destroy(plan); return rc; }
+        printf("turboFFT_sync, %d, %d, %8.3f, %8.3f, %8.3f\n", logN, (int)log2((double)bs), ms_s,
+               5.0 * N * logN * (double)bs / ms_s * 1000.0 / 1e9, N * (double)bs * (double)b.esize * 2.0 / ms_s * 1000.0 / 1e9);
+    }
     if (cfg.if_ft) {
         unsigned long long c[4] = {0, 0, 0, 0};
         turbofft_get_ft_counters(plan, &c[0], &c[1], &c[2], &c[3], nullptr, 0, nullptr);

@@ -6,6 +6,7 @@
 // from the generated registry, geometry is passed to the kernels at launch.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -191,6 +192,7 @@ struct turbofft_plan {
     int launches = 0;
     const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
     const tfft_kernel_entry* k_inv[3] = {nullptr, nullptr, nullptr};   // inverse plans: flavour of launch i (first and last differ from k)
+    const tfft_kernel_entry* k_dc[3] = {nullptr, nullptr, nullptr};    // fault-tolerant plans: delayed-batch-correction flavour of launch i (may be absent)
     int tb_gap[3] = {1, 1, 1};
     int resident[3] = {1, 1, 1};   // blocks of launch i that fit on the device at once
     size_t esize = 8;
@@ -212,7 +214,8 @@ struct turbofft_plan {
     int cksum_mode = 0;
     int xcd_chunk = -1;          // TURBOFFT_XCD_CHUNK: tiles per XCD chunk for every launch (0 = plain block order); -1 = unset
     int xcd_chunk_l[3] = {64, 64, 64};   // per launch: the plan row's value, else 64
-    unsigned long long checked = 0;   // checksum groups launched since the last reset
+    // stream of the most recent execution: the counter queries wait for it, not for the device
+    std::atomic<void*> last_stream{nullptr};
 };
 
 extern "C" {
@@ -282,6 +285,23 @@ void turbofft_plan_destroy(turbofft_plan_t* p) {
     delete p;
 }
 
+// (re)build the per-launch checksum tables in the plan's current mode and copy them to the device
+static int upload_checksum_tables(turbofft_plan* p) {
+    for (int i = 0; i < p->launches; ++i) {
+        long long Ni = 1ll << p->row.logNi(i);
+        std::vector<char> host((size_t)Ni * p->esize);
+        int rc = turbofft_build_checksum_vector(p->datatype, Ni, p->cksum_mode, host.data());
+        if (rc) return rc;
+        // device form: (re c + im c, re c - im c)
+        for (long long m = 0; m < Ni; ++m) {
+            if (p->datatype == TURBOFFT_FP32) { c32& v = ((c32*)host.data())[m]; float a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
+            else { c64& v = ((c64*)host.data())[m]; double a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
+        }
+        HIP_TRY(hipMemcpy(p->cksum[i], host.data(), host.size(), hipMemcpyHostToDevice));
+    }
+    return TURBOFFT_OK;
+}
+
 static int plan_build(turbofft_plan* p, const char* param_csv) {
     std::vector<Row> rows;
     if (param_csv) {
@@ -332,6 +352,11 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
         p->k[i] = k;
+        if (p->if_ft) {
+            p->k_dc[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 2, r.split(i) ? 1 : 0, 0, 0, 0, r.nt(i) & 3);
+            if (p->k_dc[i] && (size_t)p->k_dc[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
+                HIP_TRY(hipFuncSetAttribute(p->k_dc[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_dc[i]->lds_bytes));
+        }
         if (r.xc(i) > 0) p->xcd_chunk_l[i] = r.xc(i);
         // Inverse plans run the same launches with a component-swapping flavour of the first and
         // the last one (plain plans only; absent for a caller's CSV whose kernels were built
@@ -395,19 +420,12 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             HIP_TRY(hipMalloc(&p->tw_lo[i], host.size()));
             HIP_TRY(hipMemcpy(p->tw_lo[i], host.data(), host.size(), hipMemcpyHostToDevice));
         }
-        if (p->if_ft) {
-            long long Ni = 1ll << r.logNi(i);
-            std::vector<char> host((size_t)Ni * p->esize);
-            int rc = turbofft_build_checksum_vector(p->datatype, Ni, p->cksum_mode, host.data());
-            if (rc) return rc;
-            // device form: (re c + im c, re c - im c)
-            for (long long m = 0; m < Ni; ++m) {
-                if (p->datatype == TURBOFFT_FP32) { c32& v = ((c32*)host.data())[m]; float a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
-                else { c64& v = ((c64*)host.data())[m]; double a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
-            }
-            HIP_TRY(hipMalloc(&p->cksum[i], host.size()));
-            HIP_TRY(hipMemcpy(p->cksum[i], host.data(), host.size(), hipMemcpyHostToDevice));
-        }
+    }
+    if (p->if_ft) {
+        for (int i = 0; i < p->launches; ++i)
+            HIP_TRY(hipMalloc(&p->cksum[i], ((size_t)1 << r.logNi(i)) * p->esize));
+        int rc = upload_checksum_tables(p);
+        if (rc) return rc;
     }
     if (p->if_ft) {
         HIP_TRY(hipMalloc((void**)&p->counters, 8 * sizeof(unsigned long long)));
@@ -495,9 +513,14 @@ int turbofft_plan_set_tb_gap(turbofft_plan_t* p, int launch, int tb_gap) {
 int turbofft_set_ft_params(turbofft_plan_t* p, double err_smoothing, double err_threshold, int correct) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
+    if (correct < 0 || correct > 2) return fail(TURBOFFT_EINVAL, "correct must be 0 (detect only), 1 (recompute) or 2 (delayed batch correction)");
+    if (correct == 2)
+        for (int i = 0; i < p->launches; ++i)
+            if (!p->k_dc[i])
+                return fail(TURBOFFT_ENOPLAN, "no compiled delayed-correction kernel for launch %d of logN=%d (built for the built-in fault-tolerant plan rows)", i, p->logN);
     p->err_smoothing = err_smoothing;
     p->err_threshold = err_threshold;
-    p->correct = correct ? 1 : 0;
+    p->correct = correct;
     return TURBOFFT_OK;
 }
 
@@ -517,13 +540,32 @@ int turbofft_set_injection(turbofft_plan_t* p, int mode, int launch, int every, 
     return TURBOFFT_OK;
 }
 
+// Wait for the work the counters depend on: the stream of the plan's most recent execution
+// (other streams of the device keep running).  A stream handle that is no longer valid falls
+// back to a device-wide wait.
+static int sync_last_stream(turbofft_plan_t* p, hipStream_t* st_out) {
+    hipStream_t st = (hipStream_t)p->last_stream.load(std::memory_order_acquire);
+    hipError_t e = hipStreamSynchronize(st);
+    if (e == hipErrorInvalidHandle || e == hipErrorContextIsDestroyed || e == hipErrorInvalidResourceHandle) {
+        (void)hipGetLastError();
+        st = nullptr;
+        p->last_stream.store(nullptr, std::memory_order_release);
+        e = hipDeviceSynchronize();
+    }
+    if (e != hipSuccess) return fail(TURBOFFT_EHIP, "waiting for the plan's last execution failed: %s", hipGetErrorString(e));
+    *st_out = st;
+    return TURBOFFT_OK;
+}
+
 int turbofft_reset_ft_counters(turbofft_plan_t* p) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
-    p->checked = 0;
     if (!p->if_ft) return TURBOFFT_OK;
-    HIP_TRY(hipDeviceSynchronize());
-    HIP_TRY(hipMemset(p->counters, 0, 8 * sizeof(unsigned long long)));
-    HIP_TRY(hipMemset(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap));
+    hipStream_t st = nullptr;
+    int rc = sync_last_stream(p, &st);
+    if (rc) return rc;
+    HIP_TRY(hipMemsetAsync(p->counters, 0, 8 * sizeof(unsigned long long), st));
+    HIP_TRY(hipMemsetAsync(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap, st));
+    HIP_TRY(hipStreamSynchronize(st));
     return TURBOFFT_OK;
 }
 
@@ -532,38 +574,68 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
                              long long* flagged, int cap, int* nflagged) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     unsigned long long c[8] = {0};
+    hipStream_t st = nullptr;
     if (p->if_ft) {
-        HIP_TRY(hipDeviceSynchronize());
-        HIP_TRY(hipMemcpy(c, p->counters, sizeof c, hipMemcpyDeviceToHost));
+        int rc = sync_last_stream(p, &st);
+        if (rc) return rc;
+        HIP_TRY(hipMemcpyAsync(c, p->counters, sizeof c, hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
     }
-    if (checked) *checked = p->checked;
-    // one device counter per event class: [4] detections, [3] detections that could not be
-    // located; every located detection is recomputed while correction is switched on
+    // device counters: [0] checksum groups run (block 0 of every launch adds its grid size, so
+    // replays of a captured graph count too), [4] detections, [3] detections that could not be
+    // located; every located detection is corrected while correction is switched on
+    if (checked) *checked = c[0];
     if (detected) *detected = c[4];
     if (corrected) *corrected = p->correct ? c[4] - c[3] : 0;
     if (uncorrectable) *uncorrectable = c[3];
     int n = (int)(c[4] < (unsigned long long)p->flagged_cap ? c[4] : (unsigned long long)p->flagged_cap);
     if (n > cap) n = cap < 0 ? 0 : cap;
     if (nflagged) *nflagged = n;
-    if (flagged && n > 0) HIP_TRY(hipMemcpy(flagged, p->flagged, sizeof(long long) * 2 * n, hipMemcpyDeviceToHost));
+    if (flagged && n > 0) {
+        HIP_TRY(hipMemcpyAsync(flagged, p->flagged, sizeof(long long) * 2 * n, hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
+    }
     return TURBOFFT_OK;
 }
 
-static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev,
-                     bool inverse = false);
+int turbofft_set_checksum_mode(turbofft_plan_t* p, int mode) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
+    if (mode != 0 && mode != 1) return fail(TURBOFFT_EINVAL, "checksum mode must be 0 (exact) or 1 (reference)");
+    hipStream_t st = nullptr;
+    int rc = sync_last_stream(p, &st);      // executions in flight still read the old tables
+    if (rc) return rc;
+    p->cksum_mode = mode;
+    return upload_checksum_tables(p);
+}
+
+struct exec_opts {
+    hipEvent_t* ev = nullptr;     // launches+1 events: ev[i] before launch i, ev[launches] after the last
+    bool inverse = false;
+    bool sync_each = false;       // wait for every launch before issuing the next (the reference's timing loop)
+    void* workspace = nullptr;    // non-null: N*bs elements of intermediate storage; `out` then holds N*bs only
+};
+
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, const exec_opts& o);
 
 int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
-    return exec_impl(p, in_d, out_d, bs, stream, nullptr);
+    return exec_impl(p, in_d, out_d, bs, stream, exec_opts());
 }
 
 int turbofft_exec_inverse(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
-    return exec_impl(p, in_d, out_d, bs, stream, nullptr, true);
+    exec_opts o;
+    o.inverse = true;
+    return exec_impl(p, in_d, out_d, bs, stream, o);
 }
 
-// ev (optional): launches+1 events; ev[i] is recorded before launch i, ev[launches] after the last
-static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, hipEvent_t* ev,
-                     bool inverse) {
+static bool ranges_overlap(const void* a, size_t an, const void* b, size_t bn) {
+    const char *a0 = (const char*)a, *b0 = (const char*)b;
+    return a0 < b0 + bn && b0 < a0 + an;
+}
+
+static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, const exec_opts& o) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    const bool inverse = o.inverse;
     if (inverse) {
         if (p->if_ft) return fail(TURBOFFT_ENOPLAN, "fault-tolerant plans have no inverse kernels");
         for (int i = 0; i < p->launches; ++i)
@@ -576,16 +648,27 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     const long long N = 1ll << p->logN;
     if (N * bs > (1ll << 40)) return fail(TURBOFFT_EINVAL, "problem too large");
     const Row& r = p->row;
+    const size_t data_bytes = (size_t)N * bs * p->esize;
     char* out = (char*)out_d;
-    char* work = out + (size_t)N * bs * p->esize;
+    char* work = o.workspace ? (char*)o.workspace : out + data_bytes;
+    // The transform is out of place: the kernels read `in` while they write `out` (and a
+    // fault-tolerant plan reads a located tile a second time), and the workspace half of `out`
+    // is overwritten by the first launch of a multi-launch plan.
+    const size_t out_bytes = data_bytes * ((p->launches > 1 && !o.workspace) ? 2 : 1);
+    if (ranges_overlap(in_d, data_bytes, out, out_bytes))
+        return fail(TURBOFFT_EINVAL, "in [%p, +%zu) overlaps out [%p, +%zu): the transform is out of place%s", in_d, data_bytes,
+                    (void*)out, out_bytes, p->launches > 1 && !o.workspace ? " and out holds 2*N*bs elements (result + workspace)" : "");
+    if (o.workspace && (ranges_overlap(in_d, data_bytes, work, data_bytes) || ranges_overlap(out, data_bytes, work, data_bytes)))
+        return fail(TURBOFFT_EINVAL, "a buffer overlaps the workspace");
     // ping-pong so that the last launch writes out[0 .. N*bs)
     const void* src[3];
     void* dst[3];
     if (p->launches == 1) { src[0] = in_d; dst[0] = out; }
     else if (p->launches == 2) { src[0] = in_d; dst[0] = work; src[1] = work; dst[1] = out; }
     else { src[0] = in_d; dst[0] = out; src[1] = out; dst[1] = work; src[2] = work; dst[2] = out; }
+    p->last_stream.store(stream, std::memory_order_release);
     for (int i = 0; i < p->launches; ++i) {
-        const tfft_kernel_entry* k = inverse ? p->k_inv[i] : p->k[i];
+        const tfft_kernel_entry* k = inverse ? p->k_inv[i] : (p->correct == 2 ? p->k_dc[i] : p->k[i]);
         tfft_kargs a;
         memset(&a, 0, sizeof a);
         a.ntiles = launch_tiles(p, i, bs);
@@ -620,7 +703,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.ft.flagged = p->flagged;
             a.ft.flagged_cap = p->flagged_cap;
             a.ft.launch = i;
-            a.ft.correct = p->correct;
+            a.ft.correct = p->correct ? 1 : 0;
             int inj_l = p->inj_launch < 0 ? p->launches - 1 : p->inj_launch;
             a.ft.inj_mode = (inj_l == i) ? p->inj_mode : 0;
             a.ft.inj_every = p->inj_every;
@@ -634,18 +717,34 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         long long grid = (a.ntiles + a.thread_bs - 1) / a.thread_bs;
         if (grid < 1) continue;
         if (grid > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "grid of %lld blocks exceeds the launch limit", grid);
-        if (p->if_ft) p->checked += (unsigned long long)grid;   // one checksum group per block
         const void* in_arg = src[i];
         void* out_arg = dst[i];
         const void* tw_arg = p->tw;
         void* args[4] = {(void*)&in_arg, (void*)&out_arg, (void*)&tw_arg, (void*)&a};
-        if (ev) HIP_TRY(hipEventRecord(ev[i], (hipStream_t)stream));
+        if (o.ev) HIP_TRY(hipEventRecord(o.ev[i], (hipStream_t)stream));
         HIP_TRY(hipLaunchKernel(k->func, dim3((unsigned)grid), dim3((unsigned)k->threads), args, (size_t)k->lds_bytes,
                                 (hipStream_t)stream));
+        if (o.sync_each) HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     }
-    if (ev) HIP_TRY(hipEventRecord(ev[p->launches], (hipStream_t)stream));
+    if (o.ev) HIP_TRY(hipEventRecord(o.ev[p->launches], (hipStream_t)stream));
     return TURBOFFT_OK;
 }
+
+namespace {
+// events that are destroyed on every way out of a timing function
+struct EventSet {
+    std::vector<hipEvent_t> ev;
+    int create(int n) {
+        for (int i = 0; i < n; ++i) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreate(&e));
+            ev.push_back(e);
+        }
+        return TURBOFFT_OK;
+    }
+    ~EventSet() { for (hipEvent_t e : ev) (void)hipEventDestroy(e); }
+};
+}  // namespace
 
 int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
                            void* stream, float ms_per_launch[3]) {
@@ -655,21 +754,22 @@ int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, lo
         int rc = turbofft_exec(p, in_d, out_d, bs, stream);
         if (rc) return rc;
     }
-    hipEvent_t ev[4];
-    for (int i = 0; i < 4; ++i) HIP_TRY(hipEventCreate(&ev[i]));
-    int rc = TURBOFFT_OK;
-    for (int r = 0; r < reps && rc == TURBOFFT_OK; ++r) {
-        rc = exec_impl(p, in_d, out_d, bs, stream, ev);
-        if (rc) break;
-        if (hipEventSynchronize(ev[p->launches]) != hipSuccess) { rc = fail(TURBOFFT_EHIP, "hipEventSynchronize failed"); break; }
+    EventSet es;
+    int rc = es.create(4);
+    if (rc) return rc;
+    exec_opts o;
+    o.ev = es.ev.data();
+    for (int r = 0; r < reps; ++r) {
+        rc = exec_impl(p, in_d, out_d, bs, stream, o);
+        if (rc) return rc;
+        HIP_TRY(hipEventSynchronize(es.ev[p->launches]));
         for (int i = 0; i < p->launches; ++i) {
             float ms = 0;
-            if (hipEventElapsedTime(&ms, ev[i], ev[i + 1]) != hipSuccess) { rc = fail(TURBOFFT_EHIP, "hipEventElapsedTime failed"); break; }
+            HIP_TRY(hipEventElapsedTime(&ms, es.ev[i], es.ev[i + 1]));
             ms_per_launch[i] += ms / reps;
         }
     }
-    for (int i = 0; i < 4; ++i) (void)hipEventDestroy(ev[i]);
-    return rc;
+    return TURBOFFT_OK;
 }
 
 int turbofft_exec_host(turbofft_plan_t* p, const void* in_h, void* out_h, long long bs) {
@@ -698,30 +798,41 @@ int turbofft_exec_host(turbofft_plan_t* p, const void* in_h, void* out_h, long l
     return TURBOFFT_OK;
 }
 
-int turbofft_time(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
-                  void* stream, float* ms_per_exec) {
+static int time_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
+                     void* stream, float* ms_per_exec, bool sync_each) {
     if (!p || !ms_per_exec || reps < 1 || warmup < 0) return fail(TURBOFFT_EINVAL, "bad argument");
     hipStream_t st = (hipStream_t)stream;
+    exec_opts o;
+    o.sync_each = sync_each;
     for (int i = 0; i < warmup; ++i) {
-        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
+        int rc = exec_impl(p, in_d, out_d, bs, stream, o);
         if (rc) return rc;
     }
-    hipEvent_t t0, t1;
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
-    HIP_TRY(hipEventRecord(t0, st));
+    EventSet es;
+    int rc = es.create(2);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(es.ev[0], st));
     for (int i = 0; i < reps; ++i) {
-        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
-        if (rc) { (void)hipEventDestroy(t0); (void)hipEventDestroy(t1); return rc; }
+        rc = exec_impl(p, in_d, out_d, bs, stream, o);
+        if (rc) return rc;
+        if (sync_each) HIP_TRY(hipStreamSynchronize(st));      // main.cu:61
     }
-    HIP_TRY(hipEventRecord(t1, st));
-    HIP_TRY(hipEventSynchronize(t1));
+    HIP_TRY(hipEventRecord(es.ev[1], st));
+    HIP_TRY(hipEventSynchronize(es.ev[1]));
     float ms = 0;
-    HIP_TRY(hipEventElapsedTime(&ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
+    HIP_TRY(hipEventElapsedTime(&ms, es.ev[0], es.ev[1]));
     *ms_per_exec = ms / reps;
     return TURBOFFT_OK;
+}
+
+int turbofft_time(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
+                  void* stream, float* ms_per_exec) {
+    return time_impl(p, in_d, out_d, bs, warmup, reps, stream, ms_per_exec, false);
+}
+
+int turbofft_time_sync(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, int warmup, int reps,
+                       void* stream, float* ms_per_exec) {
+    return time_impl(p, in_d, out_d, bs, warmup, reps, stream, ms_per_exec, true);
 }
 
 }  // extern "C"
