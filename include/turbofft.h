@@ -74,6 +74,21 @@ void turbofft_plan_destroy(turbofft_plan_t* plan);
  * Stands in for the launch loop of test_turbofft (main.cu:46-49, 55-58). */
 int turbofft_exec(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs, void* stream);
 
+/* turbofft_exec for callers that can neither allocate nor spare a 2*N*bs output buffer (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): `out_d` holds
+ * N*bs elements whatever the number of launches, and the intermediate of a multi-launch plan
+ * lives in a workspace that is part of the library image (a file-scope device array of
+ * TURBOFFT_STATIC_WORKSPACE_BYTES per GPU, held until the process ends).  Same kernels and
+ * bit-identical results as turbofft_exec.  No counterpart in the reference, whose driver
+ * allocates the doubled output itself (initializeData.h:21).  Calls no allocating routine.
+ * A multi-launch plan needs N*bs*sizeof(T) <= TURBOFFT_STATIC_WORKSPACE_BYTES: larger batches
+ * return TURBOFFT_EINVAL (single-launch plans use no workspace and have no limit).  All calls
+ * on one GPU share that GPU's workspace: executions of multi-launch plans that overlap in time
+ * (two streams, two threads) race; the workspace is fully overwritten before it is read, so
+ * nothing has to be cleared between calls. */
+#define TURBOFFT_STATIC_WORKSPACE_BYTES (64ull << 20)
+int turbofft_exec_static(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs, void* stream);
+
 /* The unnormalised inverse transform, out[n] = sum_k in[k] exp(+2 pi i n k / N),
  * with the same plan, buffers and rules as turbofft_exec (turbofft_exec_inverse
  * of a turbofft_exec result is N times the input).  No counterpart in the

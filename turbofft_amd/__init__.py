@@ -23,6 +23,7 @@ LIB_PATH = os.path.join(_HERE, "libturbofft_hip.so")
 CLI_PATH = os.path.join(_HERE, "bin", "turbofft")
 
 FP32, FP64 = 0, 1
+STATIC_WORKSPACE_BYTES = 64 << 20      # TURBOFFT_STATIC_WORKSPACE_BYTES of include/turbofft.h
 _lib = None
 
 
@@ -60,6 +61,7 @@ def lib() -> C.CDLL:
     L.turbofft_plan_destroy.restype = None
     L.turbofft_exec.argtypes = [vp, vp, vp, ll, vp]
     L.turbofft_exec_inverse.argtypes = [vp, vp, vp, ll, vp]
+    L.turbofft_exec_static.argtypes = [vp, vp, vp, ll, vp]
     L.turbofft_exec_host.argtypes = [vp, vp, vp, ll]
     L.turbofft_time.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_time_sync.argtypes = [vp, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
@@ -239,6 +241,11 @@ class TurboFFT:
     # ---- execution ----
     def exec(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
         _check(lib().turbofft_exec(self._h, in_ptr, out_ptr, bs, stream))
+
+    def exec_static(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
+        """turbofft_exec with an N*bs output buffer: the intermediate of a multi-launch plan goes to
+        the library's static device workspace (STATIC_WORKSPACE_BYTES per GPU); allocates nothing."""
+        _check(lib().turbofft_exec_static(self._h, in_ptr, out_ptr, bs, stream))
 
     def exec_inverse(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):
         _check(lib().turbofft_exec_inverse(self._h, in_ptr, out_ptr, bs, stream))

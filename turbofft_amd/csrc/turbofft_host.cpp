@@ -302,6 +302,8 @@ static int upload_checksum_tables(turbofft_plan* p) {
     return TURBOFFT_OK;
 }
 
+namespace { int static_workspace(void** ptr); }
+
 static int plan_build(turbofft_plan* p, const char* param_csv) {
     std::vector<Row> rows;
     if (param_csv) {
@@ -426,6 +428,12 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             HIP_TRY(hipMalloc(&p->cksum[i], ((size_t)1 << r.logNi(i)) * p->esize));
         int rc = upload_checksum_tables(p);
         if (rc) return rc;
+    }
+    if (p->launches > 1) {
+        // look the static workspace of this device up now, so that turbofft_exec_static finds it
+        // ready (a failure is reported by that call, which tries again)
+        void* ws = nullptr;
+        if (static_workspace(&ws) != TURBOFFT_OK) g_err.clear();
     }
     if (p->if_ft) {
         HIP_TRY(hipMalloc((void**)&p->counters, 8 * sizeof(unsigned long long)));
@@ -609,6 +617,34 @@ int turbofft_set_checksum_mode(turbofft_plan_t* p, int mode) {
     return upload_checksum_tables(p);
 }
 
+// ---- the library's static device workspace (turbofft_exec_static) --------------------------
+// One array per GPU the library runs on, held until the process ends.  In host code the
+// array's name is only a handle: the device address comes from hipGetSymbolAddress, once per
+// device, and that pointer is what kernels and copies are given.
+#define TFFT_STATIC_WS_BYTES TURBOFFT_STATIC_WORKSPACE_BYTES
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[TFFT_STATIC_WS_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device (looked up on first use per device)
+int static_workspace(void** ptr) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(TURBOFFT_EINVAL, "device ordinal %d is beyond the %d this library tracks", dev, kMaxDevices);
+    void* q = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!q) {
+        hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !q)
+            return fail(TURBOFFT_EHIP, "hipGetSymbolAddress(static workspace) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev].store(q, std::memory_order_release);
+    }
+    *ptr = q;
+    return TURBOFFT_OK;
+}
+}  // namespace
+
 struct exec_opts {
     hipEvent_t* ev = nullptr;     // launches+1 events: ev[i] before launch i, ev[launches] after the last
     bool inverse = false;
@@ -625,6 +661,23 @@ int turbofft_exec(turbofft_plan_t* p, const void* in_d, void* out_d, long long b
 int turbofft_exec_inverse(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
     exec_opts o;
     o.inverse = true;
+    return exec_impl(p, in_d, out_d, bs, stream, o);
+}
+
+int turbofft_exec_static(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
+    exec_opts o;
+    if (p->launches > 1) {
+        // the intermediate of a multi-launch plan is N*bs elements
+        const unsigned long long need = ((unsigned long long)bs << p->logN) * p->esize;
+        if ((bs >> (62 - p->logN)) != 0 || need > TFFT_STATIC_WS_BYTES)
+            return fail(TURBOFFT_EINVAL, "turbofft_exec_static: %lld transforms of 2^%d points need %llu bytes of intermediate "
+                        "storage, the static workspace holds %llu; use turbofft_exec with a 2*N*bs output buffer",
+                        bs, p->logN, need, (unsigned long long)TFFT_STATIC_WS_BYTES);
+        int rc = static_workspace(&o.workspace);
+        if (rc) return rc;
+    }
     return exec_impl(p, in_d, out_d, bs, stream, o);
 }
 
