@@ -131,6 +131,20 @@ int turbofft_time_launches(turbofft_plan_t* plan, const void* in_d, void* out_d,
 int turbofft_plan_info(const turbofft_plan_t* plan, int* launches, int logNi[3], int BSi[3],
                        int ni[3], size_t lds_bytes[3], int threads[3]);
 
+/* Small batches.  The plan rows are tuned with the device full (logBS+logN = 28); a batch of
+ * a few transforms of 2^13..2^18 points would occupy a handful of CUs.  For those sizes the
+ * built-in table holds a second row of narrow tiles in two launches (param_<T>_small.csv), and
+ * a plain plan made from the built-in table runs it for bs <= turbofft_plan_small_batch_max()
+ * (0: none).  Results meet the same accuracy bar; they are not bit-identical to the large-batch
+ * row's, whose decomposition differs.  Buffers are unchanged (`out` as documented above).  For
+ * the sizes whose large-batch row is a single launch the intermediate of the two launches is a
+ * buffer the plan owns: executions of the SAME plan that overlap in time (two streams, two
+ * threads) with such a batch race on it -- use one plan per stream, or switch the small-batch
+ * row off with turbofft_plan_set_small_batch(plan, 0).  No counterpart in the reference, which
+ * has one row per size (main.cu:99,123). */
+long long turbofft_plan_small_batch_max(const turbofft_plan_t* plan);
+int turbofft_plan_set_small_batch(turbofft_plan_t* plan, int enable);
+
 /* Grid size of launch `launch` for `bs` transforms (main.cu:32). */
 long long turbofft_plan_grid(const turbofft_plan_t* plan, int launch, long long bs);
 

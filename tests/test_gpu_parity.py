@@ -540,6 +540,52 @@ def test_cli_sync_timing_line():
     assert len(a) == len(b) == 2 and all(y > 0.9 * x for x, y in zip(a, b))
 
 
+SMALL = [(dt, r) for dt in ("float2", "double2")
+         for r in __import__("turbofft_amd.codegen.plan", fromlist=["load_plan_csv"]).load_plan_csv(
+             os.path.join(os.path.dirname(turbofft_amd.LIB_PATH), "param", "gfx950", f"param_{dt}_small.csv"))]
+
+
+@pytest.mark.parametrize("dt,row", SMALL, ids=[f"{dt}-{r.logN}" for dt, r in SMALL])
+def test_small_batch_rows(dt, row):
+    # batches of a few transforms run the narrow-tile row of param_<T>_small.csv (two launches that
+    # spread one transform over many CUs); the first batch above its cap runs the large-batch row.
+    # Same accuracy bar on both sides of the switch, and through the entry point without allocation.
+    torch = _torch()
+    logN, cap = row.logN, row.tiles
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    assert plan.small_batch_max() == cap
+    cdt = torch.complex64 if dt == "float2" else torch.complex128
+    st = torch.cuda.current_stream().cuda_stream
+    for bs in sorted({1, 2, 3, cap, cap + 1}):
+        x = make(bs, 1 << logN, dt, 7 * logN + bs)
+        xd = torch.from_numpy(x).cuda()
+        ref = O.fft_ref(x)
+        guard = 1024
+        out = torch.full((plan.out_elems(bs) + guard,), 5.0 - 2.0j, dtype=cdt, device="cuda")
+        plan.exec(xd.data_ptr(), out.data_ptr(), bs, st)
+        torch.cuda.synchronize()
+        y = out[: bs << logN].view(bs, -1).cpu().numpy()
+        assert max(O.rel_l2(y[b], ref[b]) for b in range(bs)) <= O.tolerance(dt, logN), (bs, "small" if bs <= cap else "large")
+        assert bool((out[plan.out_elems(bs):] == 5.0 - 2.0j).all()), "wrote past the output buffer"
+        # without workspace from the caller
+        out2 = torch.full(((bs << logN) + guard,), 5.0 - 2.0j, dtype=cdt, device="cuda")
+        plan.exec_static(xd.data_ptr(), out2.data_ptr(), bs, st)
+        torch.cuda.synchronize()
+        assert torch.equal(out2[: bs << logN], out[: bs << logN])
+        assert bool((out2[bs << logN:] == 5.0 - 2.0j).all())
+    # switched off: the large-batch row serves every batch
+    plan.set_small_batch(False)
+    assert plan.small_batch_max() == 0
+    x = make(2, 1 << logN, dt, 3)
+    y = gpu_fft(plan, x)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    # fault-tolerant plans and caller-supplied tables keep their one row
+    ft = turbofft_amd.TurboFFT(logN, dt, if_ft=1)
+    assert ft.small_batch_max() == 0
+    ft.close()
+    plan.close()
+
+
 def test_overlapping_buffers_are_rejected():
     torch = _torch()
     for logN, dt in ((10, "float2"), (16, "float2")):

@@ -37,7 +37,13 @@ def test_registry_has_every_kernel_of_the_builtin_plans():
         for r in P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}_ft.csv")):
             assert rows[r.logN].launches > 0
             ft_rows[r.logN] = r
-        for key in collect_keys(rows, dtype, [0], inverse=True) + collect_keys(ft_rows, dtype, [1]):
+        for key in collect_keys(rows, dtype, [0], inverse=True) + collect_keys(ft_rows, dtype, [1, 2]):
+            assert key.name in have
+        # the small-batch rows: two launches of narrow tiles, column 21 = largest batch served
+        import dataclasses
+        small = P.load_plan_csv(os.path.join(ROOT, "turbofft_amd", "param", "gfx950", f"param_{dtype}_small.csv"))
+        assert small and all(r.launches == 2 and r.tiles >= 1 and rows[r.logN].launches in (1, 2) for r in small)
+        for key in collect_keys([dataclasses.replace(r, tiles=0) for r in small], dtype, [0]):
             assert key.name in have
 
 

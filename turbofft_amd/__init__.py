@@ -71,6 +71,9 @@ def lib() -> C.CDLL:
                                      C.POINTER(C.c_size_t), C.POINTER(i)]
     L.turbofft_plan_grid.argtypes = [vp, i, ll]
     L.turbofft_plan_grid.restype = ll
+    L.turbofft_plan_small_batch_max.argtypes = [vp]
+    L.turbofft_plan_small_batch_max.restype = ll
+    L.turbofft_plan_set_small_batch.argtypes = [vp, i]
     L.turbofft_plan_tb_gap.argtypes = [vp, i]
     L.turbofft_plan_set_tb_gap.argtypes = [vp, i, i]
     L.turbofft_set_ft_params.argtypes = [vp, C.c_double, C.c_double, i]
@@ -231,6 +234,13 @@ class TurboFFT:
 
     def grid(self, launch: int, bs: int) -> int:
         return lib().turbofft_plan_grid(self._h, launch, bs)
+
+    def small_batch_max(self) -> int:
+        """Largest batch that runs the narrow-tile row of the small-batch table (0: none)."""
+        return lib().turbofft_plan_small_batch_max(self._h)
+
+    def set_small_batch(self, enable: bool):
+        _check(lib().turbofft_plan_set_small_batch(self._h, int(bool(enable))))
 
     def tb_gap(self, launch: int) -> int:
         return lib().turbofft_plan_tb_gap(self._h, launch)

@@ -22,6 +22,7 @@
 
 extern "C" const char* tfft_builtin_param_csv(int datatype);   // generated: the gfx950 CSV text
 extern "C" const char* tfft_builtin_param_ft_csv(int datatype);   // generated: rows replaced in FT plans
+extern "C" const char* tfft_builtin_param_small_csv(int datatype);   // generated: rows for batches too small to fill the device
 
 namespace {
 
@@ -216,6 +217,14 @@ struct turbofft_plan {
     int xcd_chunk_l[3] = {64, 64, 64};   // per launch: the plan row's value, else 64
     // stream of the most recent execution: the counter queries wait for it, not for the device
     std::atomic<void*> last_stream{nullptr};
+    // Small batches (plain built-in plans): a second row of narrow tiles in two launches that
+    // spreads few transforms over many CUs.  `small` is a plan of its own for that row; it runs
+    // for bs <= small_max_bs.  Its intermediate lives in the upper half of the caller's `out`
+    // when this plan is a multi-launch one too, else in `small_ws` (N * small_max_bs elements).
+    turbofft_plan* small = nullptr;
+    long long small_max_bs = 0;
+    void* small_ws = nullptr;
+    bool small_enabled = true;
 };
 
 extern "C" {
@@ -275,6 +284,8 @@ const char* turbofft_kernel_name(int i) {
 
 void turbofft_plan_destroy(turbofft_plan_t* p) {
     if (!p) return;
+    if (p->small) turbofft_plan_destroy(p->small);
+    if (p->small_ws) (void)hipFree(p->small_ws);
     if (p->tw) (void)hipFree(p->tw);
     for (int i = 0; i < 3; ++i) {
         if (p->tw_lo[i]) (void)hipFree(p->tw_lo[i]);
@@ -304,6 +315,8 @@ static int upload_checksum_tables(turbofft_plan* p) {
 
 namespace { int static_workspace(void** ptr); }
 
+static int plan_build_row(turbofft_plan* p, const Row& row);
+
 static int plan_build(turbofft_plan* p, const char* param_csv) {
     std::vector<Row> rows;
     if (param_csv) {
@@ -325,7 +338,34 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     }
     if (p->logN < 1 || p->logN >= (int)rows.size() || rows[p->logN].launches() < 1 || rows[p->logN].launches() > 3)
         return fail(TURBOFFT_ENOPLAN, "no plan row for logN=%d", p->logN);
-    p->row = rows[p->logN];
+    int rc = plan_build_row(p, rows[p->logN]);
+    if (rc) return rc;
+    if (!param_csv && !p->if_ft) {
+        // the row of narrow tiles for batches that leave most of the device idle, if the
+        // built-in table has one for this size (its column 21 is the largest batch it serves)
+        std::istringstream sin(tfft_builtin_param_small_csv(p->datatype));
+        std::vector<Row> small;
+        if (!parse_csv(sin, small)) return fail(TURBOFFT_ENOPLAN, "built-in small-batch plan table is malformed");
+        for (const Row& sr : small) {
+            if (sr.logN() != p->logN || sr.launches() < 2 || sr.tiles() < 1) continue;
+            turbofft_plan* q = new turbofft_plan();
+            q->logN = p->logN; q->datatype = p->datatype; q->thread_bs = 1; q->xcd_chunk = p->xcd_chunk;
+            Row clean = sr;
+            clean.v[20] = 0;                      // column 21 is the batch cap here, not tiles per block
+            rc = plan_build_row(q, clean);
+            if (rc) { turbofft_plan_destroy(q); return rc; }
+            p->small = q;
+            p->small_max_bs = sr.tiles();
+            if (p->launches == 1)
+                HIP_TRY(hipMalloc(&p->small_ws, ((size_t)p->small_max_bs << p->logN) * p->esize));
+            break;
+        }
+    }
+    return TURBOFFT_OK;
+}
+
+static int plan_build_row(turbofft_plan* p, const Row& row) {
+    p->row = row;
     const Row& r = p->row;
     if (r.logN() != p->logN) return fail(TURBOFFT_ENOPLAN, "plan row %d describes logN=%d", p->logN, r.logN());
     p->launches = r.launches();
@@ -606,6 +646,17 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
     return TURBOFFT_OK;
 }
 
+int turbofft_plan_set_small_batch(turbofft_plan_t* p, int enable) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    p->small_enabled = enable != 0;
+    return TURBOFFT_OK;
+}
+
+long long turbofft_plan_small_batch_max(const turbofft_plan_t* p) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    return (p->small && p->small_enabled) ? p->small_max_bs : 0;
+}
+
 int turbofft_set_checksum_mode(turbofft_plan_t* p, int mode) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
@@ -668,7 +719,8 @@ int turbofft_exec_static(turbofft_plan_t* p, const void* in_d, void* out_d, long
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
     exec_opts o;
-    if (p->launches > 1) {
+    const bool small = p->small && p->small_enabled && bs <= p->small_max_bs;
+    if (p->launches > 1 || small) {
         // the intermediate of a multi-launch plan is N*bs elements
         const unsigned long long need = ((unsigned long long)bs << p->logN) * p->esize;
         if ((bs >> (62 - p->logN)) != 0 || need > TFFT_STATIC_WS_BYTES)
@@ -700,9 +752,19 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     if (!in_d || !out_d) return fail(TURBOFFT_EINVAL, "null buffer");
     const long long N = 1ll << p->logN;
     if (N * bs > (1ll << 40)) return fail(TURBOFFT_EINVAL, "problem too large");
-    const Row& r = p->row;
     const size_t data_bytes = (size_t)N * bs * p->esize;
     char* out = (char*)out_d;
+    if (p->small && p->small_enabled && bs <= p->small_max_bs && !inverse) {
+        // few transforms: the narrow-tile row, with the caller's workspace half when there is
+        // one, else the plan's own intermediate buffer
+        exec_opts so = o;
+        if (!so.workspace && p->launches == 1) so.workspace = p->small_ws;
+        if (ranges_overlap(in_d, data_bytes, out, data_bytes * ((p->launches > 1 && !o.workspace) ? 2 : 1)))
+            return fail(TURBOFFT_EINVAL, "in [%p, +%zu) overlaps out [%p, ...): the transform is out of place", in_d, data_bytes, (void*)out);
+        p->last_stream.store(stream, std::memory_order_release);
+        return exec_impl(p->small, in_d, out_d, bs, stream, so);
+    }
+    const Row& r = p->row;
     char* work = o.workspace ? (char*)o.workspace : out + data_bytes;
     // The transform is out of place: the kernels read `in` while they write `out` (and a
     // fault-tolerant plan reads a located tile a second time), and the workspace half of `out`
