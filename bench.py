@@ -241,6 +241,9 @@ def main():
     ap.add_argument("--no_vendor", action="store_true", help="skip the hipFFT side-by-side of the default line")
     ap.add_argument("--vendor", action="store_true", help="--sweep: run hipFFT after every case")
     ap.add_argument("--offline", action="store_true", help="--sweep: time the offline checksum scheme after every case")
+    ap.add_argument("--membench", action="store_true",
+                    help="time the streaming yardsticks (copy with 8- and 16-byte lanes, read only, write only) "
+                         "on 2 GiB and print one JSON line")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -254,6 +257,19 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
+    if a.membench:
+        nbytes = 2 << 30
+        src = torch.rand(nbytes // 4, device="cuda", dtype=torch.float32)
+        dst = torch.empty(nbytes // 4, device="cuda", dtype=torch.float32)
+        st = torch.cuda.current_stream().cuda_stream
+        for _ in range(20):
+            turbofft_amd.membench(0, src.data_ptr(), dst.data_ptr(), nbytes, 0, 10, st)      # clock the device up
+        res = {}
+        for mode, name, moved in ((0, "copy_8B_lanes", 2), (1, "copy_16B_lanes", 2), (2, "read_only", 1), (3, "write_only", 1)):
+            ms = sorted(turbofft_amd.membench(mode, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))
+            res[name] = {"ms_per_pass_median": ms[2], "ms_min": ms[0], "ms_max": ms[4], "GB/s": moved * nbytes / ms[2] / 1e6}
+        print(json.dumps({"membench": res, "bytes": nbytes, "tile_bytes": 65536, "threads": 256}), flush=True)
+        return 0
     if a.sweep:
         lines = []
         for dt in (0, 1):

@@ -191,8 +191,10 @@ int turbofft_set_injection(turbofft_plan_t* plan, int mode, int launch, int ever
 
 /* Counters accumulated since the last reset: groups checked, detected, corrected,
  * uncorrectable (located tile out of range); flagged[2*i] = launch, flagged[2*i+1] = tile
- * (-1 if not locatable), up to `cap` pairs; *nflagged receives the number written.  The
- * plan records at most 4096 pairs between resets: the list is truncated when *detected
+ * (-1 if not locatable), up to `cap` pairs in no particular order; *nflagged receives the
+ * number written.  The plan records at most 4096 pairs between resets, in 64 sub-lists of 64
+ * chosen by the low bits of the detecting block's index (so that a launch in which every
+ * group detects does not queue on one counter): the list is truncated when *detected
  * exceeds *nflagged.  All four counters live on the device (`checked` is added by the first
  * block of every launch), so replays of a captured HIP graph are counted.  Waits for the
  * stream of the plan's most recent turbofft_exec only, not for the device: work the caller
@@ -263,6 +265,16 @@ int turbofft_offline_checksums(int logN, int datatype, const void* in_d, const v
 int turbofft_offline_ft_time(int logN, int datatype, const void* in_d, void* out_d, long long bs,
                              int warmup, int reps, void* stream, float* ms_per_exec,
                              unsigned long long* flagged_rows);
+
+/* ---- streaming kernels of known traffic (measurement only) ----
+ * One pass over `bytes` (a multiple of 65536) in 64 KiB tiles per 256-thread block, all loads
+ * of a tile issued before its first store, timed like turbofft_time:
+ *   mode 0  copy src -> dst, 8-byte lanes      mode 1  copy, 16-byte lanes
+ *   mode 2  read src only                      mode 3  write dst only
+ * The yardsticks the FFT kernels are compared with, and kernels of known size for scaling
+ * hardware traffic counters.  No counterpart in the reference. */
+int turbofft_membench(int mode, const void* src_d, void* dst_d, size_t bytes, int warmup, int reps,
+                      void* stream, float* ms_per_pass);
 
 /* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
  * flags and output lines.  Returns the process exit code. */

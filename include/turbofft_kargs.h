@@ -14,17 +14,23 @@
 extern "C" {
 #endif
 
+#define TFFT_FT_SUB0 16            /* first sub-counter word            */
+#define TFFT_FT_SUB_STRIDE 16      /* words per sub-counter line (128 B) */
+#define TFFT_FT_COUNTER_WORDS (TFFT_FT_SUB0 + 64 * TFFT_FT_SUB_STRIDE)
+
 typedef struct tfft_ft_args {
     const void* cksum;            /* Ni entries of T: (re c + im c, re c - im c) of the input-
                                      side encoding vector c_Ni, so that re+im of x*c costs two
                                      fused multiply-adds                                      */
-    unsigned long long* counters; /* [4]=detections (also the next free slot of `flagged`),
-                                     [3]=detections whose located tile was out of range;
-                                     groups checked are counted on the host and corrected =
-                                     detected - uncorrectable while `correct` is set; [0..2] unused
-                                     [3]=uncorrectable  [4]=flagged-list length            */
-    long long* flagged;           /* flagged tile ids: flagged[2*i]=launch, [2*i+1]=tile   */
-    int flagged_cap;
+    unsigned long long* counters; /* TFFT_FT_COUNTER_WORDS words: [0] checksum groups run (added once per
+                                     launch by its first block); 64 sub-counter lines at word
+                                     TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * (block & 63): [+0] detections
+                                     (also the next free slot of that line's part of `flagged`),
+                                     [+1] detections whose located tile was out of range.  Corrected
+                                     = detected - unlocatable while `correct` is set.            */
+    long long* flagged;           /* flagged tiles as (launch, tile) pairs: sub-counter line k owns
+                                     pairs [k * cap/64, (k+1) * cap/64)                       */
+    int flagged_cap;              /* pairs in `flagged`, a multiple of 64                     */
     int launch;                   /* launch index written into `flagged`                   */
     int correct;                  /* 1: recompute the located tile (the if_err=1 variants) */
     int inj_mode;                 /* 0 none; 1 reference cadence (tile cnt == block %

@@ -35,6 +35,45 @@ class KArgs(C.Structure):
                 ("tw_hi", C.c_void_p), ("tw_lo", C.c_void_p), ("ft", FtArgs)]
 
 
+FT_SUB0, FT_SUB_STRIDE, FT_COUNTER_WORDS = 16, 16, 16 + 64 * 16      # include/turbofft_kargs.h
+
+
+class FtState:
+    """Counter block and flagged list of a fault-tolerant launch, laid out as the kernels expect
+    (64 sub-counter lines, each owning a 64th of the list), and the totals the library derives."""
+
+    def __init__(self, kargs, cap=512):
+        assert cap % 64 == 0
+        self.counters = np.zeros(FT_COUNTER_WORDS, dtype=np.uint64)
+        self.flagged = np.full(2 * cap, -7, dtype=np.int64)
+        self.cap = cap
+        kargs.ft.counters = self.counters.ctypes.data
+        kargs.ft.flagged = self.flagged.ctypes.data
+        kargs.ft.flagged_cap = cap
+
+    @property
+    def checked(self):
+        return int(self.counters[0])
+
+    @property
+    def detected(self):
+        return int(self.counters[FT_SUB0::FT_SUB_STRIDE].sum())
+
+    @property
+    def unlocatable(self):
+        return int(self.counters[FT_SUB0 + 1::FT_SUB_STRIDE].sum())
+
+    def pairs(self):
+        region = self.cap // 64
+        out = []
+        for k in range(64):
+            have = min(int(self.counters[FT_SUB0 + FT_SUB_STRIDE * k]), region)
+            for j in range(have):
+                i = k * region + j
+                out.append((int(self.flagged[2 * i]), int(self.flagged[2 * i + 1])))
+        return out
+
+
 def ctype_of(dtype):
     return np.complex64 if dtype == "float2" else np.complex128
 

@@ -25,11 +25,7 @@ def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, in
     x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
     ka = simlib.KArgs()
     ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = ntiles, bs, thread_bs, tb_gap
-    counters = np.zeros(8, dtype=np.uint64)
-    flagged = np.full(2 * 64, -7, dtype=np.int64)
-    ka.ft.counters = counters.ctypes.data
-    ka.ft.flagged = flagged.ctypes.data
-    ka.ft.flagged_cap = 64
+    st = simlib.FtState(ka)
     ka.ft.launch = 0
     ka.ft.correct = correct
     ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_s, ka.ft.inj_m, ka.ft.inj_mag = \
@@ -39,12 +35,10 @@ def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, in
     cv = O.dft_checksum_vector(N, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)      # device form of the table
     y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
-    # the kernels keep one counter per event class ([4] detections, [3] not locatable); the
-    # host derives the rest the same way the library does
-    counters[1] = counters[4]
-    counters[2] = counters[4] - counters[3] if correct else 0
-    nfl = int(counters[4])
-    fl = [(int(flagged[2 * i]), int(flagged[2 * i + 1])) for i in range(min(nfl, 64))]
+    # the kernels keep detections and unlocatable detections; the host derives the rest the same
+    # way the library does: [0] checked, [1] detected, [2] corrected, [3] uncorrectable
+    counters = [st.checked, st.detected, st.detected - st.unlocatable if correct else 0, st.unlocatable]
+    fl = st.pairs()
     return sp, x, y, counters, fl
 
 
@@ -176,31 +170,27 @@ def test_delayed_batch_correction_ragged_rows():
     x = rnd((bs, N), 9).astype(np.complex128)
     ka = simlib.KArgs()
     ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = ntiles, bs, 3, 2
-    counters = np.zeros(8, dtype=np.uint64)
-    flagged = np.full(2 * 64, -7, dtype=np.int64)
-    ka.ft.counters, ka.ft.flagged, ka.ft.flagged_cap = counters.ctypes.data, flagged.ctypes.data, 64
+    st = simlib.FtState(ka)
     ka.ft.correct, ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_mag = 1, 2, 1 << 30, ntiles - 1, 100.0
     ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
     cv = O.dft_checksum_vector(N, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
     y = simlib.run_sim(sp, x, bs * N, ka, (ntiles + 2) // 3, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
-    assert counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == ntiles - 1
+    assert st.detected == 1 and st.unlocatable == 0 and st.pairs() == [(0, ntiles - 1)]
     assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
 
 
-def _ft_args(ka, ntiles, correct, inj_tile, mag, cap=64):
-    counters = np.zeros(8, dtype=np.uint64)
-    flagged = np.full(2 * cap, -7, dtype=np.int64)
-    ka.ft.counters, ka.ft.flagged, ka.ft.flagged_cap = counters.ctypes.data, flagged.ctypes.data, cap
+def _ft_args(ka, ntiles, correct, inj_tile, mag):
+    st = simlib.FtState(ka)
     ka.ft.correct, ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_mag = correct, 2, 1 << 30, inj_tile, mag
     ka.ft.inj_s, ka.ft.inj_m = 1, 0
     ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
-    return counters, flagged
+    return st
 
 
-@pytest.mark.parametrize("ft", [1, 2])
+@pytest.mark.parametrize("ft,tbs", [(1, 3), (2, 3), (2, 1)])
 @pytest.mark.parametrize("dtype,logNi,BS,n,log_ncols", [("double2", 7, 16, 8, 8), ("float2", 8, 16, 16, 6)])
-def test_column_kernel_corrects_an_injected_tile(ft, dtype, logNi, BS, n, log_ncols):
+def test_column_kernel_corrects_an_injected_tile(ft, tbs, dtype, logNi, BS, n, log_ncols):
     # recompute (ft=1) and delayed batch correction (ft=2) in a column launch: the patch of
     # the delayed flavour is formed before the inter-launch twiddle and multiplied by it
     sp = KernelSpec(KernelKey(dtype, "col", logNi, BS, n, ft))
@@ -208,15 +198,15 @@ def test_column_kernel_corrects_an_injected_tile(ft, dtype, logNi, BS, n, log_nc
     x = rnd((outer, Ni, ncols), 5)
     ka = simlib.KArgs()
     ka.ntiles = outer * ncols // BS
-    ka.thread_bs, ka.tb_gap, ka.log_ncols = 3, 2, log_ncols
+    ka.thread_bs, ka.tb_gap, ka.log_ncols = tbs, 2, log_ncols
     lo_bits, hi, lo = simlib.split_tables(logNi + log_ncols, dtype)
     ka.tw_lo_bits = lo_bits
-    counters, flagged = _ft_args(ka, ka.ntiles, 1, 7, 1e4)
+    st = _ft_args(ka, ka.ntiles, 1, 7, 1e4)
     cv = O.dft_checksum_vector(Ni, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
-    grid = (ka.ntiles + 2) // 3
+    grid = (ka.ntiles + tbs - 1) // tbs
     y = simlib.run_sim(sp, x, x.size, ka, grid, simlib.twiddle_table(Ni, dtype), hi, lo, ck=ck).reshape(outer, Ni, ncols)
-    assert counters[0] == grid and counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == 7
+    assert st.checked == grid and st.detected == 1 and st.unlocatable == 0 and st.pairs() == [(0, 7)]
     ref = np.fft.fft(x.astype(simlib.ctype_of(dtype)).astype(np.complex128), axis=1)
     k = np.arange(Ni)[:, None]
     col = np.arange(ncols)[None, :]
@@ -224,23 +214,43 @@ def test_column_kernel_corrects_an_injected_tile(ft, dtype, logNi, BS, n, log_nc
     assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)
 
 
-@pytest.mark.parametrize("ft", [1, 2])
+@pytest.mark.parametrize("ft,tbs", [(1, 2), (2, 2), (2, 1)])
 @pytest.mark.parametrize("dtype,logA,BS,n,logQ,logC", [("double2", 8, 8, 8, 0, 4), ("float2", 8, 16, 16, 3, 4)])
-def test_transposing_kernel_corrects_an_injected_tile(ft, dtype, logA, BS, n, logQ, logC):
+def test_transposing_kernel_corrects_an_injected_tile(ft, tbs, dtype, logA, BS, n, logQ, logC):
     sp = KernelSpec(KernelKey(dtype, "rowT", logA, BS, n, ft))
     A, Q, Cc = 1 << logA, 1 << logQ, 1 << logC
     bs = 2
     x = rnd((bs, Cc, Q, A), 7)
     ka = simlib.KArgs()
     ka.ntiles = bs * Q * Cc // BS
-    ka.thread_bs, ka.tb_gap = 2, 3
+    ka.thread_bs, ka.tb_gap = tbs, 3
     ka.logQ, ka.logC, ka.logN = logQ, logC, logA + logQ + logC
-    counters, flagged = _ft_args(ka, ka.ntiles, 1, ka.ntiles - 1, 1e4)
+    st = _ft_args(ka, ka.ntiles, 1, ka.ntiles - 1, 1e4)
     cv = O.dft_checksum_vector(A, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)
-    grid = (ka.ntiles + 1) // 2
+    grid = (ka.ntiles + tbs - 1) // tbs
     y = simlib.run_sim(sp, x, x.size, ka, grid, simlib.twiddle_table(A, dtype), ck=ck).reshape(bs, A, Q, Cc)
-    assert counters[0] == grid and counters[4] == 1 and counters[3] == 0 and int(flagged[1]) == ka.ntiles - 1
+    assert st.checked == grid and st.detected == 1 and st.unlocatable == 0 and st.pairs() == [(0, ka.ntiles - 1)]
     xc = x.astype(simlib.ctype_of(dtype)).astype(np.complex128)
     ref = np.transpose(np.fft.fft(xc, axis=3), (0, 3, 2, 1))
     assert O.rel_l2(y, ref) < O.tolerance(dtype, logA)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("logNi,BS,n", [(8, 4, 16), (10, 1, 8)])
+def test_delayed_flavour_checks_a_single_tile_group_before_storing(dtype, logNi, BS, n):
+    # thread_bs = 1: every group is one tile, the reference cadence injects into every tile.  The
+    # `_fd` kernels hold such a tile in registers until it is checked and transform the saved
+    # input again when it is flagged, so the result is bit-identical to an undisturbed run.
+    ntiles = 9
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, 1, 3, inj_mode=1, correct=1, ft=2)
+    assert c[0] == ntiles and c[1] == ntiles == c[2] and c[3] == 0
+    assert sorted(t for _, t in fl) == list(range(ntiles))
+    sp, x0, y0, c0, fl0 = run_ft(dtype, logNi, BS, n, ntiles, 1, 3, inj_mode=0, correct=1, ft=2)
+    assert c0[1] == 0 and np.array_equal(x, x0) and np.array_equal(y, y0)
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+    # detect only: the held tile is stored as computed, error included
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, 1, 3, inj_mode=1, correct=0, ft=2)
+    assert c[1] == ntiles and c[2] == 0
+    err = np.abs(y - O.fft_ref(x)).reshape(ntiles, BS, -1)
+    assert np.allclose(err[:, 0, :], 100.0, rtol=1e-3) and (BS == 1 or err[:, 1:, :].max() < 1e-2)

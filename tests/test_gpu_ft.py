@@ -213,6 +213,31 @@ def test_delayed_batch_correction_matches_oracle_model(dt, logN, bs, tbs):
     plan.close()
 
 
+@pytest.mark.parametrize("dt,logN,bs", [("float2", 10, 64), ("double2", 10, 16), ("float2", 8, 512), ("double2", 16, 4), ("float2", 21, 1)])
+def test_delayed_correction_of_single_tile_groups_is_bit_identical(dt, logN, bs):
+    # thread_bs = 1 with the reference cadence: every tile of the last launch carries an error.
+    # The delayed flavour holds a one-tile group in registers until it is checked and transforms
+    # the saved input again when it is flagged: every tile is flagged and corrected, nothing is
+    # read twice, and the result equals the undisturbed run bit for bit.
+    plan = turbofft_amd.TurboFFT(logN, dt, if_err=1, thread_bs=1)
+    plan.set_ft_params(1000.0 if logN <= 10 else 0.0, 1e-3 if logN <= 10 else (1e-4 if dt == "float2" else 1e-9), correct=2)
+    plan.set_injection(1, mag=100.0 if logN <= 10 else 1e4)
+    x = make(bs, 1 << logN, dt, logN + 3)
+    y, c = run(plan, x)
+    last = plan.launches - 1
+    ntiles = plan.grid(last, bs)
+    assert c["detected"] == ntiles == c["corrected"] and c["uncorrectable"] == 0
+    if ntiles <= 4096:
+        assert sorted(c["flagged"]) == [(last, t) for t in range(ntiles)] and not c["flagged_truncated"]
+    else:
+        assert c["flagged_truncated"] and len(c["flagged"]) == 4096
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    assert c0["detected"] == 0 and np.array_equal(y, y0)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    plan.close()
+
+
 def test_delayed_batch_correction_host_chosen_tiles_and_earlier_launch():
     plan = turbofft_amd.TurboFFT(15, "double2", if_ft=1, thread_bs=2)
     plan.set_ft_params(1000.0, 1e-3, correct=2)

@@ -88,6 +88,7 @@ def lib() -> C.CDLL:
     L.turbofft_main.argtypes = [i, C.POINTER(C.c_char_p)]
     L.turbofft_vendor_exec.argtypes = [i, i, vp, vp, ll, vp]
     L.turbofft_vendor_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_membench.argtypes = [i, vp, vp, C.c_size_t, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_offline_checksums.argtypes = [i, i, vp, vp, ll, vp, vp, vp]
     L.turbofft_offline_ft_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_ulonglong)]
     _lib = L
@@ -180,6 +181,14 @@ def offline_ft_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, war
     _check(lib().turbofft_offline_ft_time(logN, _datatype(datatype), in_ptr, out_ptr, bs, warmup, reps, stream,
                                           C.byref(ms), C.byref(flagged)))
     return ms.value, flagged.value
+
+
+def membench(mode: int, src_ptr: int, dst_ptr: int, nbytes: int, warmup: int = 2, reps: int = 10, stream: int = 0) -> float:
+    """ms per pass of a streaming kernel of known traffic: 0 copy with 8-byte lanes, 1 copy with
+    16-byte lanes, 2 read only, 3 write only (measurement yardsticks, not part of any transform)."""
+    ms = C.c_float(0)
+    _check(lib().turbofft_membench(mode, src_ptr, dst_ptr, nbytes, warmup, reps, stream, C.byref(ms)))
+    return ms.value
 
 
 def turbofft_main(argv: List[str]) -> int:

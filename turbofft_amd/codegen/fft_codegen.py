@@ -530,7 +530,7 @@ class KernelEmitter:
         of the located tile; add what the tile's earlier trip stored, so that the stores that
         follow write the patched result."""
         sp = self.s
-        c("if (is_redo) {")
+        c("if (is_redo && !hold) {")
         c.ind += 1
         c(f"{self.T2} pv[{sp.n}];")
         for e, ld in enumerate(loads):
@@ -668,7 +668,9 @@ class KernelEmitter:
             # extra trip: the registers hold FFT(sum of the group's inputs); what the located tile's
             # stored result lacks is that minus the sum of the group's outputs (fft_codegen.py:401-404,
             # 427-429; the notebook's b_out += FFT(A e) - B_out e with unit weights)
-            c("else {")
+            # (a group of one tile is checked before it is stored: its extra trip simply
+            # transforms the saved input again and stores that)
+            c("else if (!hold) {")
             c.ind += 1
             for e in range(sp.n):
                 c(f"r[{self.out_reg(e)}] = csub(r[{self.out_reg(e)}], sy[{e}]);")
@@ -814,7 +816,14 @@ class KernelEmitter:
                     continue
                 if sp.ft:
                     self.emit_ft_output(c)
+                if sp.dc:
+                    # the only tile of a group is held back until the group has been checked
+                    c("if (!hold || is_redo) {")
+                    c.ind += 1
                 self.emit_store(c)
+                if sp.dc:
+                    c.ind -= 1
+                    c("}")
                 c("(void)t;")
                 out.append(("barrier", c.text()))
             else:
@@ -859,7 +868,7 @@ class KernelEmitter:
             c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
-            c("long long bx = pbx;")
+            c("long long bx = pbx; const long long pbx_raw = pbx; (void)pbx_raw;")
             LT = R if sp.split else T2
             c(f"std::vector<{LT}> ldsv({sp.lds_elems}); {LT}* lds = ldsv.data();")
             c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
@@ -874,7 +883,7 @@ class KernelEmitter:
             c(f"{LT}* lds = ({LT}*)lds_raw;")
             c("const unsigned tx = threadIdx.x;")
             c("const long long grid = gridDim.x;")
-            c("long long bx = blockIdx.x;")
+            c("long long bx = blockIdx.x; const long long pbx_raw = blockIdx.x; (void)pbx_raw;")
             c(f"{T2} r[{sp.n}];")
             if sp.pf:
                 c(f"{T2} rn[{sp.n}];")
@@ -923,6 +932,12 @@ class KernelEmitter:
             else:
                 c("if (blockIdx.x == 0 && tx == 0) atomicAdd(&a.ft.counters[0], (unsigned long long)grid);")
             c("long long redo_tile = -1; int extra = 0;")
+            if sp.dc:
+                # A group of a single tile (thread_bs = 1, or a ragged last group) is verified
+                # before its result leaves the registers: nothing is stored until the block has
+                # decided, and a flagged tile is transformed again from the input the threads
+                # still hold -- no second pass over HBM in either direction.
+                c("const bool hold = count == 1 && a.ft.correct != 0;")
             if self.ft_table_resident():
                 self.emit_ft_table_resident_load(c, sim)
             c("for (int it = 0; it < count + extra; ++it) {")
@@ -953,6 +968,16 @@ class KernelEmitter:
             self.thread_block(c, sim, ph)
         if sp.ft:
             self.emit_ft_decide(c, sim)
+            if sp.dc:
+                st = Code()
+                self.map_vars(st, sp.npass_lds - 1)
+                st("(void)x; (void)s;")
+                st("if (hold && !is_redo && !extra) {")
+                st.ind += 1
+                self.emit_store(st)
+                st.ind -= 1
+                st("}")
+                self.thread_block(c, sim, st.text())
             if sp.pf:
                 # the tile to recompute is known only now: fetch it for the extra trip
                 c("if (extra && it == count - 1) {")
@@ -1014,22 +1039,24 @@ class KernelEmitter:
         c("if (det) k = (int)round(fabs(delta2) / fabs(delta));")
         c("const bool valid = det && k >= 1 && k <= count;")
         c("const long long bad = valid ? tile0 + (long long)(k - 1) * gstride : -1;")
-        c("if (tx == 0) {")
+        c("if (tx == 0 && det) {")
         c.ind += 1
+        # One atomic per detection.  Detections are counted in 64 counters on separate cache
+        # lines, chosen by the block index, and each owns a 64th of the flagged list: a launch in
+        # which every group flags a tile (the reference's injection cadence with small groups)
+        # would otherwise queue all its blocks on one address.
+        c("const unsigned sub = (unsigned)(pbx_raw & 63);")
+        c("unsigned long long* sc = a.ft.counters + TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * sub;")
+        c("const unsigned long long region = (unsigned long long)(a.ft.flagged_cap >> 6);")
         if sim:
-            c("if (det) {")
-            c("    const unsigned long long slot = a.ft.counters[4]++;")
-            c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
-            c("    if (!valid) a.ft.counters[3] += 1;")
-            c("}")
+            c("const unsigned long long slot = sc[0]++;")
         else:
-            # one atomic per detection: the slot counter is also the detection count, and
-            # corrected = detected - uncorrectable when correction is on
-            c("if (det) {")
-            c("    const unsigned long long slot = atomicAdd(&a.ft.counters[4], 1ull);")
-            c("    if (slot < (unsigned long long)a.ft.flagged_cap) { a.ft.flagged[2 * slot] = a.ft.launch; a.ft.flagged[2 * slot + 1] = bad; }")
-            c("    if (!valid) atomicAdd(&a.ft.counters[3], 1ull);")
-            c("}")
+            c("const unsigned long long slot = atomicAdd(sc, 1ull);")
+        c("if (slot < region) { long long* fl = a.ft.flagged + 2 * (sub * region + slot); fl[0] = a.ft.launch; fl[1] = bad; }")
+        if sim:
+            c("if (!valid) sc[1] += 1;")
+        else:
+            c("if (!valid) atomicAdd(sc + 1, 1ull);")
         c.ind -= 1
         c("}")
         c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")

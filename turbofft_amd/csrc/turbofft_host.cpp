@@ -476,8 +476,8 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         if (static_workspace(&ws) != TURBOFFT_OK) g_err.clear();
     }
     if (p->if_ft) {
-        HIP_TRY(hipMalloc((void**)&p->counters, 8 * sizeof(unsigned long long)));
-        HIP_TRY(hipMemset(p->counters, 0, 8 * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void**)&p->counters, TFFT_FT_COUNTER_WORDS * sizeof(unsigned long long)));
+        HIP_TRY(hipMemset(p->counters, 0, TFFT_FT_COUNTER_WORDS * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void**)&p->flagged, sizeof(long long) * 2 * p->flagged_cap));
         HIP_TRY(hipMemset(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap));
     }
@@ -611,7 +611,7 @@ int turbofft_reset_ft_counters(turbofft_plan_t* p) {
     hipStream_t st = nullptr;
     int rc = sync_last_stream(p, &st);
     if (rc) return rc;
-    HIP_TRY(hipMemsetAsync(p->counters, 0, 8 * sizeof(unsigned long long), st));
+    HIP_TRY(hipMemsetAsync(p->counters, 0, TFFT_FT_COUNTER_WORDS * sizeof(unsigned long long), st));
     HIP_TRY(hipMemsetAsync(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap, st));
     HIP_TRY(hipStreamSynchronize(st));
     return TURBOFFT_OK;
@@ -621,28 +621,44 @@ int turbofft_get_ft_counters(turbofft_plan_t* p, unsigned long long* checked, un
                              unsigned long long* corrected, unsigned long long* uncorrectable,
                              long long* flagged, int cap, int* nflagged) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
-    unsigned long long c[8] = {0};
+    std::vector<unsigned long long> c(TFFT_FT_COUNTER_WORDS, 0ull);
     hipStream_t st = nullptr;
     if (p->if_ft) {
         int rc = sync_last_stream(p, &st);
         if (rc) return rc;
-        HIP_TRY(hipMemcpyAsync(c, p->counters, sizeof c, hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipMemcpyAsync(c.data(), p->counters, c.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
         HIP_TRY(hipStreamSynchronize(st));
     }
     // device counters: [0] checksum groups run (block 0 of every launch adds its grid size, so
-    // replays of a captured graph count too), [4] detections, [3] detections that could not be
-    // located; every located detection is corrected while correction is switched on
-    if (checked) *checked = c[0];
-    if (detected) *detected = c[4];
-    if (corrected) *corrected = p->correct ? c[4] - c[3] : 0;
-    if (uncorrectable) *uncorrectable = c[3];
-    int n = (int)(c[4] < (unsigned long long)p->flagged_cap ? c[4] : (unsigned long long)p->flagged_cap);
-    if (n > cap) n = cap < 0 ? 0 : cap;
-    if (nflagged) *nflagged = n;
-    if (flagged && n > 0) {
-        HIP_TRY(hipMemcpyAsync(flagged, p->flagged, sizeof(long long) * 2 * n, hipMemcpyDeviceToHost, st));
-        HIP_TRY(hipStreamSynchronize(st));
+    // replays of a captured graph count too); detections and detections that could not be located
+    // are spread over 64 sub-counter lines; every located detection is corrected while
+    // correction is switched on
+    unsigned long long det = 0, unloc = 0;
+    for (int k = 0; k < 64; ++k) {
+        det += c[TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * k];
+        unloc += c[TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * k + 1];
     }
+    if (checked) *checked = c[0];
+    if (detected) *detected = det;
+    if (corrected) *corrected = p->correct ? det - unloc : 0;
+    if (uncorrectable) *uncorrectable = unloc;
+    int n = 0;
+    if (flagged && cap > 0 && det > 0) {
+        // every sub-counter line owns a 64th of the list; hand the recorded pairs out in line order
+        const int region = p->flagged_cap / 64;
+        std::vector<long long> all((size_t)2 * p->flagged_cap);
+        HIP_TRY(hipMemcpyAsync(all.data(), p->flagged, all.size() * sizeof(long long), hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        for (int k = 0; k < 64 && n < cap; ++k) {
+            unsigned long long have = c[TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * k];
+            if (have > (unsigned long long)region) have = region;
+            for (unsigned long long j = 0; j < have && n < cap; ++j, ++n) {
+                flagged[2 * n] = all[2 * ((size_t)k * region + j)];
+                flagged[2 * n + 1] = all[2 * ((size_t)k * region + j) + 1];
+            }
+        }
+    }
+    if (nflagged) *nflagged = n;
     return TURBOFFT_OK;
 }
 
