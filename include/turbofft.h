@@ -145,6 +145,12 @@ int turbofft_plan_info(const turbofft_plan_t* plan, int* launches, int logNi[3],
 long long turbofft_plan_small_batch_max(const turbofft_plan_t* plan);
 int turbofft_plan_set_small_batch(turbofft_plan_t* plan, int enable);
 
+/* Name of the kernel that launch `launch` of a forward execution runs with the plan's current
+ * settings (correction scheme, checksum table, threshold); the role of reading
+ * TurboFFT_Kernel_Entry's table entry (TurboFFT.h:22-25).  For batches served by the
+ * small-batch row the kernels are that row's. */
+const char* turbofft_plan_kernel_name(const turbofft_plan_t* plan, int launch);
+
 /* Grid size of launch `launch` for `bs` transforms (main.cu:32). */
 long long turbofft_plan_grid(const turbofft_plan_t* plan, int launch, long long bs);
 
@@ -178,6 +184,16 @@ int turbofft_set_ft_params(turbofft_plan_t* plan, double err_smoothing, double e
  * replaces the tables.  The environment variable TURBOFFT_CHECKSUM_MODE=1 selects mode 1 at
  * plan creation. */
 int turbofft_set_checksum_mode(turbofft_plan_t* plan, int mode);
+/* Compact checksum table.  For some sizes the built-in fault-tolerant rows (columns 31-33 of
+ * param_<T>_ft.csv) run a kernel flavour that does not hold the complex input-side vector c_N in
+ * registers (2n per lane) but reads one real number per element: with the exact cube root,
+ * c_N[m] = kappa (1 - i cot(pi (m/N + 1/3))), kappa = (1 - rho^N)/2.  The cotangents are stored
+ * in half precision for fp32 kernels and in single precision for fp64 kernels (a quarter of the
+ * complex table), which leaves a residual of up to 1e-4 (1e-8) of the checksum magnitude on clean
+ * data: the flavour runs while err_threshold >= 5e-4 (1e-6) and the checksum mode is 0, otherwise
+ * the same launch runs its full-table flavour.  TURBOFFT_COMPACT_CHECKSUM=0 in the environment
+ * at plan creation keeps the full tables always.  The checksum arithmetic is otherwise the
+ * reference's (fft_codegen.py:354-367); it has no compact form. */
 
 /* Error injection for the launch `launch` (-1 = last, the reference's choice):
  *   mode 0  none

@@ -11,10 +11,18 @@ Parity status (what pins each function):
   twiddle_table           closed form exp(-2*pi*i*m/c)         (pinned).
   dft_checksum_vector     mode="exact": hand-computed N=2,4 vectors and the
                           geometric-series closed form          (pinned);
-                          mode="reference": reproduces the float-rounded angle
-                          of the reference table builder; only the formula in
-                          the reference pins it -> PARITY UNPINNED for the
-                          float32 libm rounding of cosf/sinf.
+                          mode="reference": the float-rounded angle of the
+                          reference table builder, pinned by an independent
+                          multiprecision evaluation of the same source lines
+                          (tests/mp_checksum.py: float32 angle via struct,
+                          cos/sin and the sum in 40-digit arithmetic; agreement
+                          to 1e-14 in fp64, to float accumulation rounding in
+                          fp32; five wrong readings of the lines -- unrounded
+                          angle, 2*pi rounded first, index product rounded
+                          first, r started at the wrong residue, +i exponent,
+                          exact sqrt(3)/2 -- are each told apart)  (pinned).
+  compact_cotangents      this build's compact form of the exact vector; pinned against
+                          the (pinned) exact mode element by element to float16 rounding.
   block_fft / plan_fft    restatement of the reference kernel algebra (DIF
                           passes, twiddle recurrences, four-step digit maps);
                           checked against fft_ref for every plan class.
@@ -151,6 +159,8 @@ def dft_checksum_vector(N: int, dtype, mode: str = "exact") -> np.ndarray:
     """c_N[i] = sum_{j<N} W_N^{ij} r[j%3]   (abft.h:21-61).
 
     mode="exact":     angles reduced exactly, accumulated in fp64, cast to T.
+    mode="compact":   this build's half-precision cotangent form of the exact vector (no
+                      counterpart in the reference): see compact_cotangents.
     mode="reference": the reference's arithmetic -- the angle 2*pi*i*j is
                       rounded to float *before* the division by float(N)
                       (abft.h:34-35, 55-56), cos/sin in T, accumulation over j
@@ -160,6 +170,10 @@ def dft_checksum_vector(N: int, dtype, mode: str = "exact") -> np.ndarray:
     if mode == "exact":
         rvec = checksum_r(np.complex128)[np.arange(N) % 3]
         return np.fft.fft(rvec).astype(ct)        # c[i] = sum_j r[j%3] W^{ij}
+    if mode == "compact":
+        # what the kernels that read the compact table multiply with: kappa (1 - i t[m]), t in
+        # half precision for fp32 kernels and in single precision for fp64 kernels
+        return (compact_kappa(N) * (1.0 - 1j * compact_cotangents(N, dtype).astype(np.float64))).astype(ct)
     if mode != "reference":
         raise ValueError(mode)
     rt = _rtype(dtype)
@@ -182,6 +196,39 @@ def dft_checksum_vector(N: int, dtype, mode: str = "exact") -> np.ndarray:
         accx = (accx + (x * rx - y * ry)).astype(rt)
         accy = (accy + (x * ry + y * rx)).astype(rt)
     return (accx.astype(np.float64) + 1j * accy.astype(np.float64)).astype(ct)
+
+
+def compact_kappa(N: int) -> complex:
+    """(1 - rho^N) / 2 for the exact cube root rho = exp(-2 pi i / 3)."""
+    return (1.0 - np.exp(-2j * np.pi * (N % 3) / 3.0)) / 2.0
+
+
+def compact_cotangents(N: int, dtype="float2") -> np.ndarray:
+    """The compact checksum table (a design of this build, not reference behaviour).
+
+    With r[j%3] = rho^j for the exact cube root rho, c_N[m] = sum_j (rho W^m)^j is a geometric
+    series: c_N[m] = (1 - rho^N) / (1 - rho W^m), and 1 / (1 - e^{-i theta}) = 1/2 - (i/2) cot(theta/2)
+    makes it kappa (1 - i t[m]) with kappa = (1 - rho^N)/2 and the single real number
+    t[m] = cot(pi (m/N + 1/3)) per element.  Stored in half precision for fp32 kernels and in
+    single precision for fp64 kernels, which bounds the usable detection threshold from below
+    (the library switches to the full table under 5e-4 and 1e-6).
+    The reference's r uses a float-rounded sqrt(3)/2, 1.6e-8 away from rho: far below float16."""
+    m = np.arange(N, dtype=np.float64)
+    a = np.pi * (3.0 * m + N) / (3.0 * N)
+    return (np.cos(a) / np.sin(a)).astype(np.float16 if _ctype(dtype) == np.complex64 else np.float32)
+
+
+def compact_table_words(N: int, n: int, dtype="float2") -> np.ndarray:
+    """Device layout of the compact table for a kernel whose threads hold n elements x + Tr*e
+    (Tr = N/n).  fp32 kernels: 32-bit word [x + Tr*q] = (t[x + Tr*2q] low half, t[x + Tr*(2q+1)]
+    high half); fp64 kernels: word [m] = t[m] in single precision."""
+    if _ctype(dtype) == np.complex128:
+        return compact_cotangents(N, dtype).view(np.uint32).copy()
+    Tr = N // n
+    bits = compact_cotangents(N).view(np.uint16).astype(np.uint32)
+    x = np.arange(Tr)[None, :]
+    q = np.arange(n // 2)[:, None]
+    return (bits[x + Tr * 2 * q] | (bits[x + Tr * (2 * q + 1)] << 16)).reshape(-1).astype(np.uint32)
 
 
 def dft_checksum_table(dtype, mode: str = "exact", max_log: int = 13) -> np.ndarray:

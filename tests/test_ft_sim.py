@@ -18,8 +18,8 @@ def rnd(shape, seed):
 
 
 def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0,
-           inj_m=0, mag=100.0, seed=0, split=0, pf=0, ft=1):
-    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, ft, split, pf))
+           inj_m=0, mag=100.0, seed=0, split=0, pf=0, ft=1, ck=0):
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, ft, split, pf, ck=ck))
     N = 1 << logNi
     bs = ntiles * BS
     x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
@@ -34,6 +34,8 @@ def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, in
     grid = (ntiles + thread_bs - 1) // thread_bs
     cv = O.dft_checksum_vector(N, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)      # device form of the table
+    if sp.ck16:
+        ck = O.compact_table_words(N, n, dtype).view(simlib.ctype_of(dtype))   # the compact table, as the buffer type the launcher passes
     y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
     # the kernels keep detections and unlocatable detections; the host derives the rest the same
     # way the library does: [0] checked, [1] detected, [2] corrected, [3] uncorrectable
@@ -254,3 +256,31 @@ def test_delayed_flavour_checks_a_single_tile_group_before_storing(dtype, logNi,
     assert c[1] == ntiles and c[2] == 0
     err = np.abs(y - O.fft_ref(x)).reshape(ntiles, BS, -1)
     assert np.allclose(err[:, 0, :], 100.0, rtol=1e-3) and (BS == 1 or err[:, 1:, :].max() < 1e-2)
+
+
+@pytest.mark.parametrize("dtype,ck", [("float2", 1), ("float2", 2), ("double2", 1), ("double2", 2)])
+@pytest.mark.parametrize("logNi,BS,n,split", [(8, 4, 16, 0), (10, 1, 8, 1), (7, 8, 8, 0)])
+def test_compact_checksum_table_flavour(dtype, ck, logNi, BS, n, split):
+    # `_h` / `_h2` kernels read one reduced-precision cotangent per element instead of a complex
+    # entry (kept in registers, or read again per tile): same decisions on the reference cadence,
+    # clean data stays clean, and the decisions equal the oracle model fed the compact vector
+    ntiles, tbs, gap = 24, 4, 3
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=1, correct=1, split=split, ck=ck)
+    groups = O.tile_groups(ntiles, tbs, gap)
+    injs = O.reference_injections(groups, tbs, 100.0)
+    assert c[1] == len(injs) == c[2] and c[3] == 0
+    assert sorted(t for _, t in fl) == sorted(i.tile for i in injs)
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+    ct = simlib.ctype_of(dtype)
+    xt = x.reshape(ntiles, BS, -1)
+    yt = O.fft_ref(xt).astype(ct)
+    for inj in injs:
+        yt[inj.tile, inj.s, :] += inj.mag
+    dec = O.ft_launch_model(xt, yt, n, groups, dtype, O.dft_checksum_vector(1 << logNi, dtype, "compact"))
+    assert sorted(d.tile for d in dec if d.detected) == sorted(t for _, t in fl)
+    sp, x, y, c, fl = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=0, correct=1, split=split, ck=ck)
+    assert c[1] == 0 and not fl and O.rel_l2(y, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+    clean = O.ft_launch_model(xt, O.fft_ref(xt).astype(ct), n, groups, dtype,
+                              O.dft_checksum_vector(1 << logNi, dtype, "compact"))
+    # the table's rounding leaves a residual well under the rule the flavour is used with
+    assert max(abs(d.delta) / (1000.0 + abs(d.mag)) for d in clean) < (2e-4 if dtype == "float2" else 1e-7)

@@ -259,6 +259,62 @@ def test_delayed_batch_correction_host_chosen_tiles_and_earlier_launch():
     plan.close()
 
 
+COMPACT = [("float2", 13, 64), ("float2", 15, 16), ("float2", 20, 2), ("float2", 22, 1), ("double2", 7, 4096), ("double2", 21, 1)]
+
+
+@pytest.mark.parametrize("dt,logN,bs", COMPACT)
+def test_compact_checksum_table_rows(dt, logN, bs):
+    # rows of the fault-tolerant table that read the compact (reduced-precision cotangent) form of
+    # the checksum vector: clean data raises nothing, an error sized above the rule is caught,
+    # located and recomputed bit-identically, decisions equal the oracle model fed the compact
+    # vector, and a rule too tight for the table's precision (or the reference's own table)
+    # runs the full-table flavour of the same launches
+    tbs = 4
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=tbs)
+    names = plan.kernel_names()
+    assert any("_h_ft" in n or "_h2_ft" in n for n in names), names
+    gaps = [7, 5, 3][:plan.launches]
+    for i, g in enumerate(gaps):
+        plan.set_tb_gap(i, g)
+    x = make(bs, 1 << logN, dt, logN + 11)
+    y, c = run(plan, x)
+    assert c["detected"] == 0 and O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    row = O.PlanRow.from_list(plan.plan_row())
+    last = plan.launches - 1
+    compact_last = "_h" in names[last]
+    clean, _ = O.ft_plan_model(x, row, dt, tbs, gaps, None, table_mode="compact" if compact_last else "exact")
+    assert max(abs(d.delta) / (1000.0 + abs(d.mag)) for d in clean[last]) < (3e-4 if dt == "float2" else 1e-6)
+    mag = float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[last])) / 0.366))
+    plan.set_ft_params(1000.0, 1e-3, correct=True)
+    plan.set_injection(1, mag=mag)
+    y1, c1 = run(plan, x)
+    groups = O.tile_groups(O.launch_geometry(row, bs)[last].ntiles, tbs, gaps[last])
+    injs = O.reference_injections(groups, tbs, mag)
+    dec, _ = O.ft_plan_model(x, row, dt, tbs, gaps, injs, table_mode="compact" if compact_last else "exact")
+    for d in dec[last]:
+        ratio = abs(d.delta) / (1000.0 + abs(d.mag)) / 1e-3
+        assert ratio < 0.67 or ratio > 1.5, "test case sits on the detection threshold"
+    model = sorted((last, d.tile) for d in dec[last] if d.detected)
+    # (for sub-FFTs of 2048 points and more the rule saturates below its threshold for
+    # single-element errors of any size: the model says whether this tile is in that regime)
+    print(f"compact rows: {len(model)} of {len(injs)} injections above the rule in the model", flush=True)
+    assert sorted(c1["flagged"]) == model and c1["corrected"] == len(model)
+    if len(model) == len(injs):
+        assert np.array_equal(y1, y)
+    # a tight rule, and the reference's own table, switch to the full-table kernels
+    plan.set_injection(0)
+    plan.set_ft_params(0.0, 1e-4 if dt == "float2" else 1e-9, correct=True)
+    tight = plan.kernel_names()
+    assert not any("_h_ft" in n or "_h2_ft" in n for n in tight), tight
+    y2, c2 = run(plan, x)
+    assert c2["detected"] == 0 and np.array_equal(y2, y)
+    plan.set_ft_params(1000.0, 1e-3, correct=True)
+    assert plan.kernel_names() == names
+    plan.set_checksum_mode("reference")
+    assert not any("_h" in n for n in plan.kernel_names())
+    plan.close()
+
+
 def test_reference_default_magnitude_is_below_the_rule_at_8192_points():
     # the model of the reference rule predicts NO detection for err_inj=100 on a
     # U[-1,1) fp32 8192-point tile (|delta| = 36.6, mag ~ 1.5e5): the GPU must agree

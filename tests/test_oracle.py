@@ -117,6 +117,35 @@ def test_checksum_reference_mode_pinned_by_multiprecision(N):
     assert 1e-6 < np.max(np.abs(o64 - b)) / np.max(np.abs(b)) < 1e-1
 
 
+@pytest.mark.parametrize("N", [64, 128, 1024, 8192])
+def test_compact_checksum_form_matches_the_exact_vector(N):
+    # kappa (1 - i cot(pi (m/N + 1/3))) is the geometric-series closed form of c_N for the exact
+    # cube root; against the exact vector (built from the float-rounded sqrt(3)/2 by an FFT) it
+    # may differ by float16 rounding of the cotangent only.  A wrong kappa for odd log2 N, a sign
+    # error in the cotangent or a shifted angle is off by O(1) relative.
+    c = O.dft_checksum_vector(N, "double2", "exact")
+    h = O.dft_checksum_vector(N, "float2", "compact").astype(np.complex128)
+    t = O.compact_cotangents(N).astype(np.float64)
+    assert np.max(np.abs(h - c) / np.abs(c)) < 6e-4 + 2e-8 * N
+    h32 = O.dft_checksum_vector(N, "double2", "compact").astype(np.complex128)      # single-precision cotangents
+    h16 = O.dft_checksum_vector(N, "float2", "compact").astype(np.complex128)       # half-precision cotangents
+    assert np.max(np.abs(h32 - c) / np.abs(c)) < 1e-7 + 2e-8 * N
+    # the cotangent alone carries the rounding: unrounded, the form is exact up to what the
+    # literal's 1.55e-8 contributes (its own pole, of height 1.55e-8 * N / pi, sits at m = N/3)
+    a = np.pi * (3.0 * np.arange(N) + N) / (3.0 * N)
+    full = O.compact_kappa(N) * (1 - 1j * np.cos(a) / np.sin(a))
+    assert np.max(np.abs(full - c) / np.abs(c)) < 2e-8 * N
+    assert np.max(np.abs(full - c)) / np.max(np.abs(c)) < 1e-7
+    assert np.all(np.isfinite(t)) and np.max(np.abs(t)) < (3 * N / np.pi) * (1 + 2 ** -10)       # largest entry, float16-rounded
+    # device layout: thread x, register pair q -> elements x + Tr*2q and x + Tr*(2q+1)
+    n = 8
+    w = O.compact_table_words(N, n)
+    Tr = N // n
+    bits = O.compact_cotangents(N).view(np.uint16)
+    for x, q in ((0, 0), (1, 0), (Tr - 1, n // 2 - 1), (3 % Tr, 1)):
+        assert w[x + Tr * q] & 0xffff == bits[x + Tr * 2 * q] and w[x + Tr * q] >> 16 == bits[x + Tr * (2 * q + 1)]
+
+
 def test_checksum_table_offsets():
     t = O.dft_checksum_table("float2", max_log=6)
     assert t.shape == (32768,)

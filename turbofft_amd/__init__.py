@@ -74,6 +74,8 @@ def lib() -> C.CDLL:
     L.turbofft_plan_small_batch_max.argtypes = [vp]
     L.turbofft_plan_small_batch_max.restype = ll
     L.turbofft_plan_set_small_batch.argtypes = [vp, i]
+    L.turbofft_plan_kernel_name.argtypes = [vp, i]
+    L.turbofft_plan_kernel_name.restype = C.c_char_p
     L.turbofft_plan_tb_gap.argtypes = [vp, i]
     L.turbofft_plan_set_tb_gap.argtypes = [vp, i, i]
     L.turbofft_set_ft_params.argtypes = [vp, C.c_double, C.c_double, i]
@@ -250,6 +252,10 @@ class TurboFFT:
 
     def set_small_batch(self, enable: bool):
         _check(lib().turbofft_plan_set_small_batch(self._h, int(bool(enable))))
+
+    def kernel_names(self) -> List[str]:
+        """Kernels the launches of a forward execution run with the current settings."""
+        return [(lib().turbofft_plan_kernel_name(self._h, i) or b"").decode() for i in range(self.launches)]
 
     def tb_gap(self, launch: int) -> int:
         return lib().turbofft_plan_tb_gap(self._h, launch)

@@ -93,6 +93,9 @@ class KernelSpec:
         self.kind = k.kind
         self.ft = bool(k.ft)
         self.dc = int(k.ft) == 2    # delayed batch correction: sums of the group's inputs and outputs per thread
+        self.ck16 = bool(k.ck)      # compact checksum table: one cotangent per element (half precision for fp32, single for fp64)
+        if self.ck16 and (int(k.ft) != 1 or k.n % 2 or k.pf):
+            raise ValueError(f"{k}: the compact checksum table is for recompute-correcting kernels without prefetch")
         self.split = bool(k.split)
         self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
         self.xl = bool(k.xl)        # last (radix 2/4/8) pass across lanes instead of through LDS
@@ -572,14 +575,27 @@ class KernelEmitter:
         instead of once per tile (-5..6 % run time).  Not under the 128-register cap of a
         1024-thread block, where the extra registers spill, nor when the entries alone would
         take more than 64 registers."""
+        if self.s.ck16:
+            return self.s.threads < 1024 and int(self.s.key.ck) == 1          # n/2 packed words per thread
         return self.s.threads < 1024 and self.s.n * (2 if self.R == "float" else 4) <= 64
+
+    def compact_kappa(self) -> Tuple[float, float]:
+        """kappa = (1 - rho^Ni) / 2 with rho = exp(-2 pi i / 3): Ni = 1 (mod 3) for even log2 Ni,
+        2 (mod 3) for odd."""
+        k = ilog2(self.s.Ni) % 2 + 1
+        ang = -2.0 * math.pi * k / 3.0
+        return (1.0 - math.cos(ang)) / 2.0, -math.sin(ang) / 2.0
 
     def emit_ft_table_resident_load(self, c: Code, sim: bool):
         sp = self.s
         pre = Code()
         self.map_vars(pre, 0)
-        for e in range(sp.n):
-            pre(f"cvr[{e}] = {self.TWLU}(ck, {sp.Tr * e}u, x);")
+        if sp.ck16:
+            for q in range(sp.n // 2 if self.R == "float" else sp.n):
+                pre(f"cwr[{q}] = CKW(ck, {sp.Tr * q}u, x);")
+        else:
+            for e in range(sp.n):
+                pre(f"cvr[{e}] = {self.TWLU}(ck, {sp.Tr * e}u, x);")
         pre("(void)s;")
         c("if (count > 0) {")
         c.ind += 1
@@ -606,7 +622,42 @@ class KernelEmitter:
         # two independent multiply-add chains (one per component): two operations per element;
         # a single `acc += a*b + c*d` costs three, since the sum may not be reassociated
         c(f"{self.R} acc = 0, acy = 0;")
-        if self.ft_table_resident():
+        if sp.ck16:
+            # Compact table.  With the exact cube root rho the input-side vector has the closed form
+            #   c[m] = (1 - rho^Ni) / (1 - rho W^m) = kappa (1 - i t[m]),  t[m] = cot(pi (m/Ni + 1/3)),
+            # so one real number per element carries it: re+im of x c = kp*(sum x.re + sum t x.im)
+            # + kq*(sum x.im - sum t x.re) with kp, kq = re kappa +- im kappa.  fp32 kernels store t in
+            # half precision, two elements of a thread per 32-bit word (word [x + Tr*q] holds elements
+            # x + Tr*2q and x + Tr*(2q+1)): 16 KiB for 8192 points, a quarter of the complex table;
+            # fp64 kernels store it in single precision, one word per element.  Small enough to be
+            # read again for every tile, or cheap enough to keep (n/2 or n registers per thread).
+            kr, ki = self.compact_kappa()
+            c(f"{self.R} sa = 0, sb = 0, sc = 0, sd = 0;")
+            B = 8
+            half = self.R == "float"       # fp32: two half-precision values per word; fp64: one float per word
+            W = sp.n // 2 if half else sp.n
+            def use(word: str, q: int):
+                if half:
+                    for h, e in ((0, 2 * q), (1, 2 * q + 1)):
+                        c(f"{{ const float tt = CKH({word}, {h}); sa += r[{e}].x; sb += r[{e}].y; sc += tt * r[{e}].y; sd += tt * r[{e}].x; }}")
+                else:
+                    c(f"{{ const double tt = (double)CKF({word}); sa += r[{q}].x; sb += r[{q}].y; sc += tt * r[{q}].y; sd += tt * r[{q}].x; }}")
+            if self.ft_table_resident():
+                for q in range(W):
+                    use(f"cwr[{q}]", q)
+            else:
+                c(f"unsigned cw[{B}];")
+                for b0 in range(0, W, B):
+                    hi = min(W, b0 + B)
+                    for q in range(b0, hi):
+                        c(f"cw[{q - b0}] = CKW(ck, {sp.Tr * q}u, xc);")
+                    c("SCHED_FENCE();")
+                    for q in range(b0, hi):
+                        use(f"cw[{q - b0}]", q)
+                    c("SCHED_FENCE();")
+            c(f"acc = {self.lit(kr + ki)} * (sa + sc) + {self.lit(kr - ki)} * (sb - sd);")
+            c("(void)acy;")
+        elif self.ft_table_resident():
             for e in range(sp.n):
                 c(f"acc += r[{e}].x * cvr[{e}].x; acy += r[{e}].y * cvr[{e}].y;")
         else:
@@ -623,7 +674,8 @@ class KernelEmitter:
                 for e in range(b0, min(sp.n, b0 + B)):
                     c(f"acc += r[{e}].x * cv[{e - b0}].x; acy += r[{e}].y * cv[{e - b0}].y;")
                 c("SCHED_FENCE();")
-        c("acc += acy;")
+        if not sp.ck16:
+            c("acc += acy;")
         c("fin1 += acc; fin2 += cntf * acc;")
         if sp.dc:
             # per-thread sum of the group's inputs (fft_codegen.py:355-357), taken before the injection
@@ -865,7 +917,7 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; unsigned cwr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx; const long long pbx_raw = pbx; (void)pbx_raw;")
@@ -890,7 +942,7 @@ class KernelEmitter:
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
                 if self.ft_table_resident():
-                    c(f"{T2} cvr[{sp.n}];")
+                    c(f"unsigned cwr[{sp.n // 2 if R == 'float' else sp.n}];" if sp.ck16 else f"{T2} cvr[{sp.n}];")
                 if sp.dc:
                     c(f"{T2} sx[{sp.n}], sy[{sp.n}];")
                     c(f"for (int e = 0; e < {sp.n}; ++e) {{ sx[e] = czero(sx[e]); sy[e] = czero(sy[e]); }}")
@@ -1005,8 +1057,8 @@ class KernelEmitter:
         if sim:
             c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
             c.ind += 1
-            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
-            c("(void)r; (void)rn; (void)cvr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& cwr = ts[tx].cwr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
+            c("(void)r; (void)rn; (void)cvr; (void)cwr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
         else:
             c("{")
             c.ind += 1
@@ -1091,7 +1143,7 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     kinds = {"row1": 0, "col": 1, "rowT": 2}
     for sp in specs:
         k = sp.key
-        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {int(k.wv)}, {int(k.nt)}, {int(k.inv)}, {sp.threads}, {sp.lds_bytes}}},')
+        c(f'    {{"{sp.name}", (const void*){sp.name}, {0 if k.dtype == "float2" else 1}, {kinds[k.kind]}, {k.logNi}, {k.BS}, {k.n}, {int(k.ft)}, {int(k.split)}, {int(k.pf)}, {int(k.xl)}, {int(k.wv)}, {int(k.nt)}, {int(k.inv)}, {int(k.ck)}, {sp.threads}, {sp.lds_bytes}}},')
     c("};")
     c('extern "C" const tfft_kernel_entry* tfft_kernel_table(int* count) {')
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")
@@ -1107,7 +1159,12 @@ def collect_keys(rows: Sequence[PlanRow], dtype: str, ft_variants: Sequence[int]
         if row.launches == 0:
             continue
         for ft in ft_variants:
-            for k in kernels_for_row(row, dtype, ft):
+            ks = kernels_for_row(row, dtype, ft)
+            if ft == 1 and any(row.ck):
+                # a launch that reads the compact checksum table also needs its full-table flavour
+                # (tight detection rules and the reference's own table run that one)
+                ks = ks + kernels_for_row(row, dtype, ft, compact=False)
+            for k in ks:
                 if k not in seen:
                     seen.add(k)
                     keys.append(k)

@@ -38,6 +38,9 @@ class PlanRow:
     wv: Tuple[int, ...] = ()         # optional columns 22-24: wavefronts per SIMD to compile for (0 = free)
     nt: Tuple[int, ...] = ()         # optional columns 25-27, tile access policy: +1 non-temporal tile loads, +2 non-temporal stores, +4 raised wave priority while the loads are issued
     xc: Tuple[int, ...] = ()         # optional columns 28-30: consecutive tiles per XCD (run time only; 0 = 64)
+    ck: Tuple[int, ...] = ()         # optional columns 31-33: the fault-tolerant kernel of the launch reads the compact
+                                     # (half-precision cotangent) form of the checksum table (fp32 only): 1 = words kept in
+                                     # registers by blocks of fewer than 1024 threads, 2 = read again for every tile
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -52,7 +55,8 @@ class PlanRow:
         ext3 = (row[17:20] + [0, 0, 0])[:3]
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
                     tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
-                    tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]), tuple((row[27:30] + [0, 0, 0])[:L]))
+                    tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]), tuple((row[27:30] + [0, 0, 0])[:L]),
+                    tuple((row[30:33] + [0, 0, 0])[:L]))
         if any(t not in range(8) for t in p.nt):
             raise ValueError(f"tile access policy columns must be 0..7 in row {row}")
         if L and sum(p.logNi) != p.logN:
@@ -82,12 +86,15 @@ class KernelKey:
     inv: int = 0     # 1: the flavour an inverse plan uses in this position -- re and im exchanged as
                      # they are loaded (row1, col as first launch) and/or before they are stored
                      # (row1, rowT): inverse = swap . forward . swap
+    ck: int = 0      # > 0: fault-tolerant fp32 kernel that reads the compact checksum table (one half-precision
+                     # cotangent per element, two per 32-bit word); 1: the words stay in registers for the tiles
+                     # of a block where the block has fewer than 1024 threads, 2: they are read again for every tile
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:
@@ -97,7 +104,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:30] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:33] if t.strip()]))
     return rows
 
 
@@ -105,9 +112,11 @@ def launch_kinds(launches: int) -> List[str]:
     return {1: ["row1"], 2: ["col", "rowT"], 3: ["col", "col", "rowT"]}[launches]
 
 
-def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False) -> List[KernelKey]:
+def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False, compact: bool = True) -> List[KernelKey]:
     """Kernels of the row's launches; with `inverse` the first and the last launch use their
-    component-swapping flavour (plain plans only), launches in between are the forward ones."""
+    component-swapping flavour (plain plans only), launches in between are the forward ones.
+    `compact`: honour the row's compact-checksum-table columns (recompute-correcting fp32
+    fault-tolerant kernels only); False gives the full-table flavour of the same launches."""
     if inverse and ft:
         raise ValueError("inverse plans have no fault-tolerant flavour")
     last = row.launches - 1
@@ -118,10 +127,12 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False) ->
                       (int(row.xl[i]) if row.xl else 0) if not ft else 0,
                       # the register budget hint was tuned on the plain kernel only (fault-tolerant
                       # kernels keep their table in registers and spill under any tighter budget)
-                      (int(row.wv[i]) if row.wv else 0) if not ft else 0,
+                      # (the compact-table flavour is the exception: its budget is tuned with it)
+                      (int(row.wv[i]) if row.wv else 0) if (not ft or (compact and int(ft) == 1 and row.ck and int(row.ck[i]))) else 0,
                       # the priority bit was timed on the plain kernel only
                       (int(row.nt[i]) & (3 if ft else 7)) if row.nt else 0,
-                      1 if inverse and i in (0, last) else 0)
+                      1 if inverse and i in (0, last) else 0,
+                      int(row.ck[i]) if (compact and int(ft) == 1 and row.ck and int(row.ck[i])) else 0)
             for i, kind in enumerate(launch_kinds(row.launches))]
 
 

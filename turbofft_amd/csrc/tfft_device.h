@@ -98,6 +98,15 @@ __device__ __forceinline__ void tfft_gstn(double2* p, double2 v) {
 #define TWLDU(p, c, i) tfft_bld<0>((p), (unsigned)(i) * TFFT_ESZ(p), (unsigned)(c) * TFFT_ESZ(p))
 #define LLD(i) (lds[(i)])
 #define LST(i, v) (lds[(i)] = (v))
+// compact checksum table: one 32-bit word holds two half-precision values
+typedef _Float16 tfft_h2v __attribute__((ext_vector_type(2)));
+#define CKW(p, c, i) (((const unsigned*)(p))[(c) + (i)])
+__device__ __forceinline__ float tfft_ckh(unsigned w, int hi) {
+    const tfft_h2v h = __builtin_bit_cast(tfft_h2v, w);
+    return hi ? (float)h.y : (float)h.x;
+}
+#define CKH(w, hi) tfft_ckh((w), (hi))
+#define CKF(w) __uint_as_float(w)
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
 // tile-independent table reads inside the tile loop instead of hoisted into registers
 #define OPAQUE(v) asm volatile("" : "+v"(v))
@@ -107,6 +116,7 @@ __device__ __forceinline__ void tfft_gstn(double2* p, double2 v) {
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 struct float2 { float x, y; };
 struct double2 { double x, y; };
@@ -138,6 +148,20 @@ extern long long tfft_sim_errors;
 #define TWLDU(p, c, i) ((p)[TFFT_CHK((long long)(c) + (long long)(i), p##_limit, #p)])
 #define OPAQUE(v)
 #define SCHED_FENCE()
+// compact checksum table (ck_limit counts complex elements of the buffer the launcher passed)
+#define CKW(p, c, i) (((const unsigned*)(p))[TFFT_CHK((long long)(c) + (long long)(i), (long long)(sizeof(*(p)) / 4) * ck_limit, "compact checksum table")])
+static inline float tfft_ckh(unsigned w, int hi) {
+    const unsigned h = hi ? (w >> 16) : (w & 0xffffu);
+    const unsigned sgn = (h >> 15) & 1u, ex = (h >> 10) & 31u, man = h & 1023u;
+    float v;
+    if (ex == 0) v = std::ldexp((float)man, -24);
+    else if (ex == 31) v = man ? NAN : INFINITY;
+    else v = std::ldexp((float)(man | 1024u), (int)ex - 25);
+    return sgn ? -v : v;
+}
+#define CKH(w, hi) tfft_ckh((w), (hi))
+static inline float tfft_ckf(unsigned w) { float f; memcpy(&f, &w, sizeof f); return f; }
+#define CKF(w) tfft_ckf(w)
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
 // cross-lane fetch in the lock-step flavour: the partner's registers as snapshotted

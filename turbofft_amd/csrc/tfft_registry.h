@@ -18,6 +18,7 @@ typedef struct tfft_kernel_entry {
     int wv;              // > 0: compiled for this many wavefronts per SIMD
     int nt;              // bit 0: non-temporal tile loads, bit 1: non-temporal tile stores, bit 2: raised wave priority for the tile loads
     int inv;             // 1: component-swapping flavour for the first / last launch of an inverse plan
+    int ck;              // 1: reads the compact (half-precision cotangent) checksum table
     int threads;         // block size
     int lds_bytes;       // dynamic LDS
 } tfft_kernel_entry;

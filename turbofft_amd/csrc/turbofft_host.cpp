@@ -61,14 +61,20 @@ namespace {
     } while (0)
 
 constexpr double kPi = 3.14159265358979323846;
+// smallest err_threshold the compact checksum tables serve: half-precision entries (fp32 kernels)
+// leave up to 1e-4 of the checksum magnitude as residual on clean data, single-precision ones
+// (fp64 kernels) 1e-8
+constexpr double kCompactMinThreshold32 = 5e-4, kCompactMinThreshold64 = 1e-6;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[30];           // 11 reference columns + optional per-launch flags: split exchange,
+    int v[33];           // 11 reference columns + optional per-launch flags: split exchange,
                          // prefetch, cross-lane last pass; then the tiles-per-block hint, the
                          // per-launch wavefronts-per-SIMD the plain kernel was compiled for and
                          // the per-launch non-temporal access bits, then the per-launch
-                         // number of consecutive tiles an XCD works on (0 = 64)
+                         // number of consecutive tiles an XCD works on (0 = 64), then the per-launch
+                         // compact-checksum-table flag of the fault-tolerant fp32 kernel
+    int ck(int i) const { return v[30 + i]; }
     int nt(int i) const { return v[24 + i]; }
     int xc(int i) const { return v[27 + i]; }
     int tiles() const { return v[20]; }
@@ -94,7 +100,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 30 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 33 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -106,12 +112,12 @@ int kind_of_launch(int launches, int i) {   // 0 row1, 1 col, 2 rowT
     return i == launches - 1 ? 2 : 1;
 }
 
-const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv, int nt, int inv = 0) {
+const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, int n, int ft, int split, int pf, int xl, int wv, int nt, int inv = 0, int ck = 0) {
     int cnt = 0;
     const tfft_kernel_entry* t = tfft_kernel_table(&cnt);
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
-            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt && t[i].inv == inv)
+            t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt && t[i].inv == inv && t[i].ck == ck)
             return &t[i];
     return nullptr;
 }
@@ -194,6 +200,8 @@ struct turbofft_plan {
     const tfft_kernel_entry* k[3] = {nullptr, nullptr, nullptr};
     const tfft_kernel_entry* k_inv[3] = {nullptr, nullptr, nullptr};   // inverse plans: flavour of launch i (first and last differ from k)
     const tfft_kernel_entry* k_dc[3] = {nullptr, nullptr, nullptr};    // fault-tolerant plans: delayed-batch-correction flavour of launch i (may be absent)
+    const tfft_kernel_entry* k_full[3] = {nullptr, nullptr, nullptr};  // where k[i] reads the compact checksum table: the flavour with the full table
+    void* cksum16[3] = {nullptr, nullptr, nullptr};                    // compact checksum tables (half-precision cotangents), launches whose k[i] reads one
     int tb_gap[3] = {1, 1, 1};
     int resident[3] = {1, 1, 1};   // blocks of launch i that fit on the device at once
     size_t esize = 8;
@@ -225,6 +233,7 @@ struct turbofft_plan {
     long long small_max_bs = 0;
     void* small_ws = nullptr;
     bool small_enabled = true;
+    bool compact_enabled = true;      // TURBOFFT_COMPACT_CHECKSUM=0 keeps the full-table kernels
 };
 
 extern "C" {
@@ -290,6 +299,7 @@ void turbofft_plan_destroy(turbofft_plan_t* p) {
     for (int i = 0; i < 3; ++i) {
         if (p->tw_lo[i]) (void)hipFree(p->tw_lo[i]);
         if (p->cksum[i]) (void)hipFree(p->cksum[i]);
+        if (p->cksum16[i]) (void)hipFree(p->cksum16[i]);
     }
     if (p->counters) (void)hipFree(p->counters);
     if (p->flagged) (void)hipFree(p->flagged);
@@ -309,6 +319,34 @@ static int upload_checksum_tables(turbofft_plan* p) {
             else { c64& v = ((c64*)host.data())[m]; double a = v.x + v.y, b = v.x - v.y; v.x = a; v.y = b; }
         }
         HIP_TRY(hipMemcpy(p->cksum[i], host.data(), host.size(), hipMemcpyHostToDevice));
+        if (p->k[i] && p->k[i]->ck) {
+            // compact form (exact angles only): t[m] = cot(pi (m/Ni + 1/3)) in half precision, two
+            // elements of a thread per word: word [x + Tr*q] = (t[x + Tr*2q], t[x + Tr*(2q+1)])
+            const long long Tr = Ni / p->row.n(i);
+            auto cot = [&](long long m) { const double a = kPi * (double)(3 * m + Ni) / (double)(3 * Ni); return cos(a) / sin(a); };
+            std::vector<unsigned> words;
+            if (p->datatype == TURBOFFT_FP32) {
+                auto half_bits = [&](long long m) -> unsigned {
+                    const _Float16 h = (_Float16)(float)cot(m);
+                    unsigned short b;
+                    memcpy(&b, &h, sizeof b);
+                    return b;
+                };
+                words.resize((size_t)(Ni / 2));
+                for (long long q = 0; q < p->row.n(i) / 2; ++q)
+                    for (long long x = 0; x < Tr; ++x)
+                        words[(size_t)(x + Tr * q)] = half_bits(x + Tr * 2 * q) | (half_bits(x + Tr * (2 * q + 1)) << 16);
+            } else {
+                // fp64 kernels: single precision, one word per element, natural order
+                words.resize((size_t)Ni);
+                for (long long m = 0; m < Ni; ++m) {
+                    const float f = (float)cot(m);
+                    memcpy(&words[(size_t)m], &f, sizeof f);
+                }
+            }
+            if (!p->cksum16[i]) HIP_TRY(hipMalloc(&p->cksum16[i], words.size() * sizeof(unsigned)));
+            HIP_TRY(hipMemcpy(p->cksum16[i], words.data(), words.size() * sizeof(unsigned), hipMemcpyHostToDevice));
+        }
     }
     return TURBOFFT_OK;
 }
@@ -393,6 +431,16 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         if (!k)
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
+        p->k_full[i] = k;
+        if (p->if_ft && r.ck(i)) {
+            // the row asks for the flavour that reads the compact checksum table; the full-table
+            // flavour stays available for the table modes and thresholds the compact form cannot serve
+            const tfft_kernel_entry* kc = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 1, r.split(i) ? 1 : 0, 0, 0, r.wv(i), r.nt(i) & 3, 0, r.ck(i));
+            if (!kc) return fail(TURBOFFT_ENOPLAN, "no compiled compact-checksum kernel for launch %d of logN=%d", i, p->logN);
+            if ((size_t)kc->lds_bytes > (size_t)prop.sharedMemPerBlock)
+                HIP_TRY(hipFuncSetAttribute(kc->func, hipFuncAttributeMaxDynamicSharedMemorySize, kc->lds_bytes));
+            k = kc;
+        }
         p->k[i] = k;
         if (p->if_ft) {
             p->k_dc[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 2, r.split(i) ? 1 : 0, 0, 0, 0, r.nt(i) & 3);
@@ -414,6 +462,8 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         }
         if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
             HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
+        if (p->k_full[i] != k && (size_t)p->k_full[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
+            HIP_TRY(hipFuncSetAttribute(p->k_full[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_full[i]->lds_bytes));
         int nb = 0;
         HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k->func, k->threads, k->lds_bytes));
         if (nb < 1) return fail(TURBOFFT_ENOPLAN, "kernel %s does not fit on a CU (LDS %d B)", k->name, k->lds_bytes);
@@ -498,6 +548,8 @@ turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_
     if (p->if_err) { p->inj_mode = 1; p->correct = 1; }   // the if_err=1 kernels inject and correct
     const char* env = getenv("TURBOFFT_CHECKSUM_MODE");
     if (env && atoi(env) == 1) p->cksum_mode = 1;
+    env = getenv("TURBOFFT_COMPACT_CHECKSUM");
+    if (env && atoi(env) == 0) p->compact_enabled = false;
     env = getenv("TURBOFFT_XCD_CHUNK");
     if (env) p->xcd_chunk = atoi(env) > 0 ? atoi(env) : 0;
     if (plan_build(p, param_csv) != TURBOFFT_OK) {
@@ -749,6 +801,22 @@ int turbofft_exec_static(turbofft_plan_t* p, const void* in_d, void* out_d, long
     return exec_impl(p, in_d, out_d, bs, stream, o);
 }
 
+// the kernel launch i runs with the plan's current settings
+static const tfft_kernel_entry* launch_kernel(const turbofft_plan* p, int i, bool inverse) {
+    const tfft_kernel_entry* k = inverse ? p->k_inv[i] : (p->correct == 2 ? p->k_dc[i] : p->k[i]);
+    // The compact checksum table holds exact-angle entries in reduced precision: tighter
+    // detection rules and the reference's own table run the full-table flavour of the launch.
+    if (k && k->ck && (p->cksum_mode != 0 || !p->compact_enabled ||
+                       p->err_threshold < (p->datatype == TURBOFFT_FP32 ? kCompactMinThreshold32 : kCompactMinThreshold64))) k = p->k_full[i];
+    return k;
+}
+
+const char* turbofft_plan_kernel_name(const turbofft_plan_t* p, int launch) {
+    if (!p || launch < 0 || launch >= p->launches) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
+    const tfft_kernel_entry* k = launch_kernel(p, launch, false);
+    return k ? k->name : nullptr;
+}
+
 static bool ranges_overlap(const void* a, size_t an, const void* b, size_t bn) {
     const char *a0 = (const char*)a, *b0 = (const char*)b;
     return a0 < b0 + bn && b0 < a0 + an;
@@ -799,7 +867,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     else { src[0] = in_d; dst[0] = out; src[1] = out; dst[1] = work; src[2] = work; dst[2] = out; }
     p->last_stream.store(stream, std::memory_order_release);
     for (int i = 0; i < p->launches; ++i) {
-        const tfft_kernel_entry* k = inverse ? p->k_inv[i] : (p->correct == 2 ? p->k_dc[i] : p->k[i]);
+        const tfft_kernel_entry* k = launch_kernel(p, i, inverse);
         tfft_kargs a;
         memset(&a, 0, sizeof a);
         a.ntiles = launch_tiles(p, i, bs);
@@ -829,7 +897,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.logQ = p->launches == 3 ? r.logNi(1) : 0;
         }
         if (p->if_ft) {
-            a.ft.cksum = p->cksum[i];
+            a.ft.cksum = k->ck ? p->cksum16[i] : p->cksum[i];
             a.ft.counters = p->counters;
             a.ft.flagged = p->flagged;
             a.ft.flagged_cap = p->flagged_cap;
