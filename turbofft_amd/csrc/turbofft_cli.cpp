@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <cmath>
 #include <complex>
 #include <cstdio>
@@ -229,7 +230,16 @@ int test_turbofft(const ProgramConfig& cfg, int logN, long long bs, int ntest, B
     float ms = 0;
     int rc = TURBOFFT_OK;
     if (cfg.if_err && cfg.ft_correction == 2) rc = turbofft_set_ft_params(plan, 1000.0, 1e-3, 2);
-    if (!rc) rc = turbofft_time(plan, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms);
+    // One warm-up execution as in the reference (main.cu:46-49), then -- for the timed sweeps --
+    // as many more as fill 30 ms: the device clocks down while a plan is being made, and ten
+    // timed executions of a sub-millisecond transform would otherwise be measured on the ramp.
+    int warm = 1;
+    if (!rc && ntest > 1) {
+        float est = 0;
+        rc = turbofft_time(plan, b.in_d, b.out_d, bs, 1, 2, nullptr, &est);
+        if (!rc && est > 0) warm = std::max(1, std::min(2000, (int)(30.0f / est)));
+    }
+    if (!rc) rc = turbofft_time(plan, b.in_d, b.out_d, bs, warm, ntest, nullptr, &ms);
     if (rc) { printf("turboFFT, %d: %s\n", logN, turbofft_last_error()); turbofft_plan_destroy(plan); return rc; }
     double N = (double)(1ll << logN);
     double gflops = 5.0 * N * logN * (double)bs / ms * 1000.0 / 1e9;             // main.cu:68
@@ -259,7 +269,14 @@ int test_turbofft(const ProgramConfig& cfg, int logN, long long bs, int ntest, B
 // test_cufft (cufft/cufft.h:14-56): the vendor library on the same buffers, same metric line
 int test_vendor_fft(const ProgramConfig& cfg, int logN, long long bs, int ntest, Buffers& b, std::vector<char>* result) {
     float ms = 0;
-    int rc = turbofft_vendor_time(logN, cfg.datatype, b.in_d, b.out_d, bs, 1, ntest, nullptr, &ms);
+    int warm = 1;
+    int rc = TURBOFFT_OK;
+    if (ntest > 1) {              // the same 30 ms of warm-up as for this library's plans
+        float est = 0;
+        rc = turbofft_vendor_time(logN, cfg.datatype, b.in_d, b.out_d, bs, 1, 2, nullptr, &est);
+        if (!rc && est > 0) warm = std::max(1, std::min(2000, (int)(30.0f / est)));
+    }
+    if (!rc) rc = turbofft_vendor_time(logN, cfg.datatype, b.in_d, b.out_d, bs, warm, ntest, nullptr, &ms);
     if (rc) { printf("hipFFT, %d: %s\n", logN, turbofft_last_error()); return rc; }
     double N = (double)(1ll << logN);
     double gflops = 5.0 * N * logN * (double)bs / ms * 1000.0 / 1e9;             // cufft.h:41
