@@ -151,27 +151,36 @@ def test_input_is_not_modified():
 
 
 def test_config2_full_size_fp32_2p13():
-    # benchmark configuration 2 at full size (2^28 points): sampled batches against the oracle,
-    # plus linearity of the whole batch as a size-independent property
+    # benchmark configuration 2 at full size (2^28 points): numpy default_rng(0), uniform[-1,1) drawn in
+    # fp64 and cast (re then im, per chunk of 1024 transforms); 64 batches spread over the set against
+    # the fp64 oracle, plus Parseval over the whole set as a size-independent property
     torch = _torch()
     logN, bs = 13, 1 << 15
     N = 1 << logN
     plan = turbofft_amd.TurboFFT(logN, "float2")
-    g = torch.Generator(device="cuda").manual_seed(0)
-    x = (torch.rand((bs, N, 2), generator=g, device="cuda", dtype=torch.float32) * 2 - 1)
-    x = torch.view_as_complex(x)
+    rng = np.random.default_rng(0)
+    x = torch.empty((bs, N), dtype=torch.complex64, device="cuda")
+    idx = sorted(set(range(0, bs, bs // 63)) | {bs - 1})[:64]
+    keep = {}
+    chunk = 1024
+    for c0 in range(0, bs, chunk):
+        part = (rng.uniform(-1, 1, (chunk, N)) + 1j * rng.uniform(-1, 1, (chunk, N))).astype(np.complex64)
+        for i in idx:
+            if c0 <= i < c0 + chunk:
+                keep[i] = part[i - c0].copy()
+        x[c0:c0 + chunk].copy_(torch.from_numpy(part))
     y = plan.fft(x)
     torch.cuda.synchronize()
-    idx = [0, 1, 777, bs // 2, bs - 1]
-    xs = x[idx].cpu().numpy()
     ys = y[idx].cpu().numpy()
-    ref = O.fft_ref(xs)
-    for i in range(len(idx)):
-        assert O.rel_l2(ys[i], ref[i]) <= O.tolerance("float2", logN)
+    ref = O.fft_ref(np.stack([keep[i] for i in idx]))
+    worst = max(O.rel_l2(ys[k], ref[k]) for k in range(len(idx)))
+    print(f"config 2: {len(idx)} sampled transforms, worst rel-L2 {worst:.3e} (bar {O.tolerance('float2', logN):.1e})", flush=True)
+    assert worst <= O.tolerance("float2", logN)
     # Parseval over the whole set: sum |X|^2 = N sum |x|^2
     ex = float((x.real.double() ** 2 + x.imag.double() ** 2).sum())
     ey = float((y.real.double() ** 2 + y.imag.double() ** 2).sum())
     assert abs(ey / (N * ex) - 1) < 1e-5
+    plan.close()
 
 
 def _full_size_check(torch, plan, dt, logN, bs, normal):
