@@ -151,8 +151,11 @@ PF = [("row1", "float2", 10, 1, 16, 0), ("row1", "double2", 7, 8, 8, 0), ("row1"
 
 @pytest.mark.parametrize("kind,dtype,logNi,BS,n,split", PF)
 @pytest.mark.parametrize("tbs", [1, 4])
-def test_prefetch_row1(kind, dtype, logNi, BS, n, split, tbs):
-    sp = KernelSpec(KernelKey(dtype, kind, logNi, BS, n, 0, split, 1))
+@pytest.mark.parametrize("pf", [1, 3])
+def test_prefetch_row1(kind, dtype, logNi, BS, n, split, tbs, pf):
+    # pf = 1: the whole next tile is fetched ahead; pf = 3: only a thread's first three elements,
+    # issued at the start of the tile's last pass
+    sp = KernelSpec(KernelKey(dtype, kind, logNi, BS, n, 0, split, pf))
     N = 1 << logNi
     bs = BS * 9 + BS // 2
     x = rnd((bs, N), logNi + 70)

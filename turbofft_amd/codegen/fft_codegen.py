@@ -98,6 +98,11 @@ class KernelSpec:
             raise ValueError(f"{k}: the compact checksum table is for recompute-correcting kernels without prefetch")
         self.split = bool(k.split)
         self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
+        # pf > 1: only the first pf elements of a thread are fetched ahead, and only from the start
+        # of the tile's last pass on (for 1024-thread blocks, which have no room for a whole set)
+        self.pfk = int(k.pf) if int(k.pf) > 1 else 0
+        if self.pfk and (k.kind != "row1" or int(k.ft) or k.xl or self.pfk >= k.n or (k.BS == 1 and k.n and False)):
+            raise ValueError(f"{k}: partial prefetch is for plain single-launch kernels, fewer elements than n")
         self.xl = bool(k.xl)        # last (radix 2/4/8) pass across lanes instead of through LDS
         self.lds_esize = self.esize // 2 if self.split else self.esize   # bytes per LDS access
         self.passes = radix_passes(self.Ni, self.n)
@@ -425,9 +430,28 @@ class KernelEmitter:
                  "rowT": ["ctl", "ct", "qd", "tb", "ubase_in", "ls", "ubase_out", "gstep"]}[sp.kind]
         c(" ".join(f"(void){n}{sfx};" for n in names))
 
-    def emit_load(self, c: Code, dst: str = "r", sfx: str = ""):
+    def emit_load(self, c: Code, dst: str = "r", sfx: str = "", elems: Optional[Sequence[int]] = None):
+        """Loads of a tile's elements into dst[e]; `elems` restricts them to some of a thread's
+        elements (row1 kernels, one element per access)."""
         sp = self.s
         lNi = ilog2(sp.Ni)
+        if elems is not None:
+            assert sp.kind == "row1" and not self.pair_access() and not int(sp.key.inv)
+            c(f"const unsigned gi{sfx} = (s << {lNi}) + x;")
+            if sp.BS > 1:
+                c(f"if ((row0{sfx} + s) < a.nrows) {{")
+                c.ind += 1
+            for e in elems:
+                c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
+            if sp.BS > 1:
+                c.ind -= 1
+                c("} else {")
+                c.ind += 1
+                for e in elems:
+                    c(f"{dst}[{e}] = czero({dst}[0]);")
+                c.ind -= 1
+                c("}")
+            return
         if sp.kind == "row1":
             c(f"const unsigned gi{sfx} = (s << {lNi}) + x;")
             if sp.BS > 1:
@@ -806,7 +830,16 @@ class KernelEmitter:
             c = Code()
             self.map_vars(c, q)
             c(f"{self.T2} t;")
-            if q == 0:
+            if q == 0 and sp.pfk:
+                # the first pfk elements were fetched during the previous tile's last pass
+                for e in range(sp.pfk):
+                    c(f"r[{e}] = rn[{e}];")
+                c("{")
+                c.ind += 1
+                self.emit_load(c, "r", "", elems=range(sp.pfk, sp.n))
+                c.ind -= 1
+                c("}")
+            elif q == 0:
                 if sp.pf:
                     # this tile's elements were fetched during the previous tile; start the
                     # fetch of the next one now so it overlaps every pass of this tile
@@ -847,6 +880,15 @@ class KernelEmitter:
                     if sp.ft:
                         self.emit_ft_input(c)
             else:
+                if sp.pfk and q == sp.npass_lds - 1:
+                    # start on the next tile while this one runs its last pass: a 1024-thread block
+                    # is alone on its CU and would otherwise have nothing in flight while it computes
+                    c("if (has_next) {")
+                    c.ind += 1
+                    self.emit_tile_decode(c, "tile_n", "_n")
+                    self.emit_load(c, "rn", "_n", elems=range(sp.pfk))
+                    c.ind -= 1
+                    c("}")
                 self.emit_lds_read(c, q, ".y" if sp.split else "")
             self.emit_pass_compute(c, q)
             if q == sp.npass_lds - 1:
@@ -938,7 +980,7 @@ class KernelEmitter:
             c("long long bx = blockIdx.x; const long long pbx_raw = blockIdx.x; (void)pbx_raw;")
             c(f"{T2} r[{sp.n}];")
             if sp.pf:
-                c(f"{T2} rn[{sp.n}];")
+                c(f"{T2} rn[{sp.pfk or sp.n}];")
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
                 if self.ft_table_resident():
@@ -973,7 +1015,7 @@ class KernelEmitter:
             self.emit_tile_decode(c, "tile0", "_n")
             pre = Code()
             self.map_vars(pre, 0)
-            self.emit_load(pre, "rn", "_n")
+            self.emit_load(pre, "rn", "_n", elems=range(sp.pfk) if sp.pfk else None)
             self.thread_block(c, sim, pre.text())
             c.ind -= 1
             c("}")

@@ -79,7 +79,8 @@ class KernelKey:
                      # checksums with delayed batch correction (per-thread sums of the group's inputs and
                      # outputs, the located tile is patched with FFT(sum x) - sum y)
     split: int = 0   # 1: every LDS exchange moves re and im in two rounds through a half-size buffer
-    pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed
+    pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed;
+                     # k > 1: only the first k elements of a thread, from the start of the tile's last pass on
     xl: int = 0      # 1: the last pass (radix 2, 4 or 8) runs across lanes (DPP / ds_swizzle), no LDS exchange
     wv: int = 0      # > 0: compiled to fit this many wavefronts per SIMD (register budget 512 / wv)
     nt: int = 0      # bit 0: tile loads are non-temporal, bit 1: tile stores are, bit 2: raised wave priority while the tile loads are issued (plain kernels)
@@ -93,7 +94,7 @@ class KernelKey:
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
-        return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf else "") + ("_x" if self.xl else "")
+        return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf == 1 else (f"_p{self.pf}" if self.pf else "")) + ("_x" if self.xl else "")
                 + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
 
 
@@ -121,7 +122,8 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False, co
         raise ValueError("inverse plans have no fault-tolerant flavour")
     last = row.launches - 1
     return [KernelKey(dtype, kind, row.logNi[i], row.BS[i], row.n[i], int(ft), int(row.split[i]) if row.split else 0,
-                      int(row.pf[i]) if row.pf else 0,
+                      # (partial prefetch, pf > 1, exists for the plain forward kernel only)
+                      (int(row.pf[i]) if (int(row.pf[i]) <= 1 or not (ft or (inverse and i in (0, last)))) else 0) if row.pf else 0,
                       # fault-tolerant plans keep the LDS path: the checksum model fixes which
                       # outputs a thread owns
                       (int(row.xl[i]) if row.xl else 0) if not ft else 0,

@@ -425,7 +425,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
     long long twN = 1;
     for (int i = 0; i < p->launches; ++i) {
         int kind = kind_of_launch(p->launches, i);
-        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
+        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, (p->if_ft && r.pf(i) > 1) ? 0 : r.pf(i),
                                                  (r.xl(i) && !p->if_ft) ? 1 : 0,    // FT plans keep the LDS path
                                                  p->if_ft ? 0 : r.wv(i), p->if_ft ? (r.nt(i) & 3) : r.nt(i));   // wave budget and priority bit: plain kernels only
         if (!k)
@@ -453,7 +453,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         // without them, and then turbofft_exec_inverse reports it).
         p->k_inv[i] = k;
         if (!p->if_ft && (i == 0 || i == p->launches - 1)) {
-            p->k_inv[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 0, r.split(i) ? 1 : 0, r.pf(i) ? 1 : 0,
+            p->k_inv[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 0, r.split(i) ? 1 : 0, r.pf(i) > 1 ? 0 : r.pf(i),
                                       r.xl(i) ? 1 : 0, r.wv(i), r.nt(i), 1);
             if (p->k_inv[i] && (size_t)p->k_inv[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
                 HIP_TRY(hipFuncSetAttribute(p->k_inv[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_inv[i]->lds_bytes));
