@@ -76,11 +76,15 @@ def stats(v):
 
 
 def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if_err=0, thread_bs=1, param=None,
-             x=None, out=None, prewarm_s=0.0, correct=None):
+             x=None, out=None, prewarm_s=0.0, correct=None, inj_every=0, inj_mag=100.0):
     N = 1 << logN
     plan = turbofft_amd.TurboFFT(logN, datatype, if_ft=if_ft, if_err=if_err, thread_bs=thread_bs, param_csv=param)
     if correct is not None:
         plan.set_ft_params(1000.0, 1e-3, correct)
+    if inj_every > 0:
+        # host-chosen cadence: one tile in every `inj_every` of the last launch gets `inj_mag` added to an element
+        plan.set_ft_params(1000.0, 1e-3, 1 if correct is None else correct)
+        plan.set_injection(2, every=inj_every, tile_phase=min(123, inj_every - 1), s=0, m=0, mag=inj_mag)
     cdt = torch.complex64 if datatype == 0 else torch.complex128
     if x is None:
         x = make_input(torch, bs, N, datatype)
@@ -230,6 +234,9 @@ def main():
     ap.add_argument("--prewarm_s", type=float, default=1.0,
                     help="seconds of untimed executions before the warm-up steps (reported as prewarm_s)")
     ap.add_argument("--correct", type=int, default=None, help="with --if_err: 1 recompute, 2 delayed batch correction")
+    ap.add_argument("--inj_every", type=int, default=0,
+                    help="with --if_ft 1: inject into one tile of every N of the last launch (host-chosen cadence) and correct")
+    ap.add_argument("--inj_mag", type=float, default=100.0, help="magnitude of the --inj_every injections")
     ap.add_argument("--no_cpu", action="store_true")
     ap.add_argument("--cpu_seconds", type=float, default=10.0)
     ap.add_argument("--sweep", action="store_true")
@@ -325,7 +332,7 @@ def main():
     logN, dt = a.logN, a.datatype
     bs = a.bs or (1 << (28 - logN))
     r, x, out = run_case(torch, turbofft_amd, logN, dt, bs, a.steps, a.warmup, a.if_ft, a.if_err, a.thread_bs, a.param,
-                         prewarm_s=a.prewarm_s, correct=a.correct)
+                         prewarm_s=a.prewarm_s, correct=a.correct, inj_every=a.inj_every, inj_mag=a.inj_mag)
     for _ in range(a.calib_copy):
         out.view(-1)[: x.numel()].copy_(x.view(-1))          # reads and writes x.numel()*sizeof(T) bytes
     torch.cuda.synchronize()
@@ -366,7 +373,8 @@ def main():
         "config": {"workload": f"forward C2C FFT {tname} N=2^{logN} batch=2^{int(math.log2(bs))} "
                                f"({launches}-launch plan {r['plan']['logNi']}, BS {r['plan']['BS']}, n {r['plan']['n']})"
                                + (", fault tolerant" if (a.if_ft or a.if_err) else ""),
-                   "logN": logN, "bs": bs, "if_ft": a.if_ft, "if_err": a.if_err, "thread_bs": a.thread_bs},
+                   "logN": logN, "bs": bs, "if_ft": a.if_ft, "if_err": a.if_err, "thread_bs": a.thread_bs,
+                   "inj_every": a.inj_every, "inj_mag": a.inj_mag if a.inj_every else None},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((dt, logN, bs, int(bool(a.if_ft or a.if_err)))),
