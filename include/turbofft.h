@@ -103,7 +103,14 @@ int turbofft_exec_inverse(turbofft_plan_t* plan, const void* in_d, void* out_d, 
 
 /* Same, from and to host memory (allocates device buffers, copies, runs,
  * synchronises, frees).  Stands in for initializeData's H2D copy plus the
- * D2H copy at main.cu:72. */
+ * D2H copy at main.cu:72.  A plain plan whose batch exceeds one piece (64 MiB
+ * of input; TURBOFFT_HOST_PIECE_BYTES in the environment overrides) streams
+ * the batch through three device slots on three streams of its own: copies in,
+ * kernels and copies out overlap when the host buffers are page-locked
+ * (hipHostMalloc), and the device memory needed is three pieces, not the
+ * batch.  The result has the bits of turbofft_exec on the whole batch.
+ * Fault-tolerant plans run the batch in one piece (tile groups and flagged
+ * tile numbers refer to the batch as passed). */
 int turbofft_exec_host(turbofft_plan_t* plan, const void* in_h, void* out_h, long long bs);
 
 /* Timed runs with HIP events on `stream`: `warmup` untimed executions, then

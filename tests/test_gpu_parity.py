@@ -130,6 +130,34 @@ def test_exec_host_matches_device_path():
     assert O.rel_l2(a, O.fft_ref(x)) <= O.tolerance("double2", 15)
 
 
+@pytest.mark.parametrize("dt,logN,bs,piece", [("float2", 10, 1000, 96), ("double2", 15, 11, 2), ("float2", 17, 7, 3),
+                                              ("float2", 23, 3, 1), ("double2", 6, 5000, 4999)])
+def test_exec_host_streams_the_batch_in_pieces(dt, logN, bs, piece, monkeypatch):
+    """Host buffers larger than one piece go through three device slots on three streams; the
+    result is that of the device path, bit for bit, for pageable and for page-locked buffers,
+    with a ragged last piece and with more pieces than slots."""
+    torch = _torch()
+    x = make(bs, 1 << logN, dt, 40 + logN)
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    want = gpu_fft(plan, x)
+    monkeypatch.setenv("TURBOFFT_HOST_PIECE_BYTES", str(piece * x.shape[1] * x.itemsize))
+    assert np.array_equal(plan.fft_host(x), want)
+    tdt = torch.complex64 if dt == "float2" else torch.complex128
+    xin = torch.empty(x.shape, dtype=tdt, pin_memory=True)
+    xin.copy_(torch.from_numpy(x))
+    out = torch.zeros(x.shape, dtype=tdt, pin_memory=True)
+    for _ in range(2):                                   # the second call reuses nothing of the first
+        plan.exec_host(xin.data_ptr(), out.data_ptr(), bs)
+        assert np.array_equal(out.numpy(), want)
+        out.zero_()
+    # a fault-tolerant plan is transformed in one piece: its groups and flagged tiles refer to the whole batch
+    if logN == 10:
+        ft = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=4)
+        assert np.array_equal(ft.fft_host(x), gpu_fft(ft, x))
+        c = ft.ft_counters()
+        assert c["checked"] == 2 * ft.grid(0, bs) and c["detected"] == 0      # two executions of the whole batch
+
+
 def test_empty_batch_and_bad_shapes():
     torch = _torch()
     plan = turbofft_amd.TurboFFT(10, "float2")

@@ -227,7 +227,8 @@ class TurboFFT:
 
     def close(self):
         if getattr(self, "_h", None):
-            lib().turbofft_plan_destroy(self._h)
+            if lib is not None:                     # (module globals are gone at interpreter shutdown)
+                lib().turbofft_plan_destroy(self._h)
             self._h = None
 
     __del__ = close
@@ -296,12 +297,17 @@ class TurboFFT:
         (self.exec_inverse if _inverse else self.exec)(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream(x.device).cuda_stream)
         return out.view(-1)[: bs * self.N].view(bs, self.N)
 
+    def exec_host(self, in_ptr: int, out_ptr: int, bs: int):
+        """turbofft_exec_host on raw host addresses (N*bs elements each; page-locked buffers let the
+        copies in, the kernels and the copies out overlap)."""
+        _check(lib().turbofft_exec_host(self._h, in_ptr, out_ptr, bs))
+
     def fft_host(self, x: np.ndarray) -> np.ndarray:
         x = np.ascontiguousarray(x, dtype=self.cdtype)
         if x.ndim != 2 or x.shape[1] != self.N:
             raise ValueError(f"expected shape (bs, {self.N}), got {x.shape}")
         out = np.empty_like(x)
-        _check(lib().turbofft_exec_host(self._h, x.ctypes.data, out.ctypes.data, x.shape[0]))
+        self.exec_host(x.ctypes.data, out.ctypes.data, x.shape[0])
         return out
 
     def time(self, in_ptr: int, out_ptr: int, bs: int, warmup: int = 1, reps: int = 10, stream: int = 0) -> float:

@@ -769,6 +769,7 @@ struct exec_opts {
     bool inverse = false;
     bool sync_each = false;       // wait for every launch before issuing the next (the reference's timing loop)
     void* workspace = nullptr;    // non-null: N*bs elements of intermediate storage; `out` then holds N*bs only
+    bool main_row = false;        // run the plan's own row whatever the batch (pieces of a larger batch)
 };
 
 static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, const exec_opts& o);
@@ -838,7 +839,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     if (N * bs > (1ll << 40)) return fail(TURBOFFT_EINVAL, "problem too large");
     const size_t data_bytes = (size_t)N * bs * p->esize;
     char* out = (char*)out_d;
-    if (p->small && p->small_enabled && bs <= p->small_max_bs && !inverse) {
+    if (p->small && p->small_enabled && bs <= p->small_max_bs && !inverse && !o.main_row) {
         // few transforms: the narrow-tile row, with the caller's workspace half when there is
         // one, else the plan's own intermediate buffer
         exec_opts so = o;
@@ -971,29 +972,114 @@ int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, lo
     return TURBOFFT_OK;
 }
 
+namespace {
+// device buffers, streams and events of one host-buffer execution, released on every way out
+struct HostPipe {
+    turbofft_plan_t* plan = nullptr;       // its last-execution stream must not outlive the streams below
+    std::vector<void*> dev;
+    std::vector<hipStream_t> st;
+    EventSet ev;
+    int alloc(void** q, size_t bytes) {
+        if (hipMalloc(q, bytes) != hipSuccess) return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes);
+        dev.push_back(*q);
+        return TURBOFFT_OK;
+    }
+    int stream(hipStream_t* q) {
+        HIP_TRY(hipStreamCreateWithFlags(q, hipStreamNonBlocking));
+        st.push_back(*q);
+        return TURBOFFT_OK;
+    }
+    ~HostPipe() {
+        for (hipStream_t q : st) (void)hipStreamSynchronize(q);   // nothing may still use the buffers
+        if (plan && !st.empty()) plan->last_stream.store(nullptr, std::memory_order_release);
+        for (hipStream_t q : st) (void)hipStreamDestroy(q);
+        for (void* q : dev) (void)hipFree(q);
+    }
+};
+
+// Transforms the whole batch in one piece: the path of fault-tolerant plans (their tile groups
+// and the tile numbers of the flagged list refer to the batch as the caller passed it) and of
+// batches that are a single piece anyway.
+int exec_host_whole(turbofft_plan_t* p, const void* in_h, void* out_h, long long bs, size_t bytes) {
+    HostPipe hp;
+    void *in_d = nullptr, *out_d = nullptr;
+    int rc = hp.alloc(&in_d, bytes);
+    if (rc) return rc;
+    rc = hp.alloc(&out_d, bytes * (p->launches > 1 ? 2 : 1));
+    if (rc) return rc;
+    HIP_TRY(hipMemcpy(in_d, in_h, bytes, hipMemcpyHostToDevice));
+    rc = turbofft_exec(p, in_d, out_d, bs, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(out_h, out_d, bytes, hipMemcpyDeviceToHost));
+    return TURBOFFT_OK;
+}
+
+size_t host_piece_bytes() {
+    // bytes of input one piece of the streamed host path carries (TURBOFFT_HOST_PIECE_BYTES overrides)
+    if (const char* e = std::getenv("TURBOFFT_HOST_PIECE_BYTES")) {
+        long long v = std::atoll(e);
+        if (v > 0) return (size_t)v;
+    }
+    return (size_t)64 << 20;       // timed 32-256 MiB with page-locked buffers: 64 MiB pieces were fastest
+}
+}  // namespace
+
 int turbofft_exec_host(turbofft_plan_t* p, const void* in_h, void* out_h, long long bs) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (bs < 0) return fail(TURBOFFT_EINVAL, "negative batch");
     if (bs == 0) return TURBOFFT_OK;
     if (!in_h || !out_h) return fail(TURBOFFT_EINVAL, "null buffer");
-    size_t bytes = ((size_t)1 << p->logN) * (size_t)bs * p->esize;
-    void *in_d = nullptr, *out_d = nullptr;
-    if (hipMalloc(&in_d, bytes) != hipSuccess) return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes);
-    if (hipMalloc(&out_d, bytes * (p->launches > 1 ? 2 : 1)) != hipSuccess) {
-        (void)hipFree(in_d);
-        return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes * 2);
+    const size_t one = ((size_t)1 << p->logN) * p->esize;            // bytes of one transform
+    const size_t bytes = one * (size_t)bs;
+    long long piece = (long long)(host_piece_bytes() / one);
+    if (piece < 1) piece = 1;
+    if (p->if_ft || p->if_err || piece >= bs) return exec_host_whole(p, in_h, out_h, bs, bytes);
+
+    // Plain plan, several pieces: the batch streams through three slots of device memory.
+    // One stream copies pieces in, one runs the plan on them in order (so nothing the plan
+    // owns is used by two executions at once), one copies results out; events hand a slot
+    // from stage to stage.  With page-locked host buffers the two copy directions and the
+    // kernels overlap; pageable buffers make each copy call block the host, which still
+    // bounds the device memory to the three slots.
+    const int kSlots = 3;
+    const long long pieces = (bs + piece - 1) / piece;
+    const int slots = pieces < kSlots ? (int)pieces : kSlots;
+    const size_t pbytes = one * (size_t)piece;
+    HostPipe hp;
+    hp.plan = p;
+    hipStream_t s_in, s_run, s_out;
+    int rc;
+    if ((rc = hp.stream(&s_in)) || (rc = hp.stream(&s_run)) || (rc = hp.stream(&s_out))) return rc;
+    void *in_d[kSlots] = {}, *out_d[kSlots] = {};
+    for (int i = 0; i < slots; ++i) {
+        if ((rc = hp.alloc(&in_d[i], pbytes))) return rc;
+        if ((rc = hp.alloc(&out_d[i], pbytes * (p->launches > 1 ? 2 : 1)))) return rc;
     }
-    int rc = TURBOFFT_OK;
-    hipError_t e = hipMemcpy(in_d, in_h, bytes, hipMemcpyHostToDevice);
-    if (e == hipSuccess) {
-        rc = turbofft_exec(p, in_d, out_d, bs, nullptr);
-        if (rc == TURBOFFT_OK) e = hipDeviceSynchronize();
-        if (rc == TURBOFFT_OK && e == hipSuccess) e = hipMemcpy(out_h, out_d, bytes, hipMemcpyDeviceToHost);
+    if ((rc = hp.ev.create(3 * slots))) return rc;
+    hipEvent_t* copied = hp.ev.ev.data();                              // piece is in in_d[slot]
+    hipEvent_t* ran = copied + slots;                                  // in_d[slot] consumed, out_d[slot] holds the result
+    hipEvent_t* drained = ran + slots;                                 // out_d[slot] is on the host
+    exec_opts eo;
+    // every piece runs the kernels the whole batch would run on the device path: the same bits
+    eo.main_row = !(p->small && p->small_enabled && bs <= p->small_max_bs);
+    for (long long c = 0; c < pieces; ++c) {
+        const int k = (int)(c % slots);
+        const long long b0 = c * piece, nb = (bs - b0 < piece) ? bs - b0 : piece;
+        const char* src = (const char*)in_h + (size_t)b0 * one;
+        char* dst = (char*)out_h + (size_t)b0 * one;
+        if (c >= slots) HIP_TRY(hipStreamWaitEvent(s_in, ran[k], 0));
+        HIP_TRY(hipMemcpyAsync(in_d[k], src, one * (size_t)nb, hipMemcpyHostToDevice, s_in));
+        HIP_TRY(hipEventRecord(copied[k], s_in));
+        HIP_TRY(hipStreamWaitEvent(s_run, copied[k], 0));
+        if (c >= slots) HIP_TRY(hipStreamWaitEvent(s_run, drained[k], 0));
+        if ((rc = exec_impl(p, in_d[k], out_d[k], nb, s_run, eo))) return rc;
+        HIP_TRY(hipEventRecord(ran[k], s_run));
+        HIP_TRY(hipStreamWaitEvent(s_out, ran[k], 0));
+        HIP_TRY(hipMemcpyAsync(dst, out_d[k], one * (size_t)nb, hipMemcpyDeviceToHost, s_out));
+        HIP_TRY(hipEventRecord(drained[k], s_out));
     }
-    (void)hipFree(in_d);
-    (void)hipFree(out_d);
-    if (rc != TURBOFFT_OK) return rc;
-    if (e != hipSuccess) return fail(TURBOFFT_EHIP, "HIP error: %s", hipGetErrorString(e));
+    HIP_TRY(hipStreamSynchronize(s_out));
     return TURBOFFT_OK;
 }
 
