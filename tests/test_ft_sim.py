@@ -258,7 +258,7 @@ def test_delayed_flavour_checks_a_single_tile_group_before_storing(dtype, logNi,
     assert np.allclose(err[:, 0, :], 100.0, rtol=1e-3) and (BS == 1 or err[:, 1:, :].max() < 1e-2)
 
 
-@pytest.mark.parametrize("dtype,ck", [("float2", 1), ("float2", 2), ("double2", 1), ("double2", 2)])
+@pytest.mark.parametrize("dtype,ck", [("float2", 1), ("float2", 2), ("float2", 3), ("double2", 1), ("double2", 2), ("double2", 3)])
 @pytest.mark.parametrize("logNi,BS,n,split", [(8, 4, 16, 0), (10, 1, 8, 1), (7, 8, 8, 0)])
 def test_compact_checksum_table_flavour(dtype, ck, logNi, BS, n, split):
     # `_h` / `_h2` kernels read one reduced-precision cotangent per element instead of a complex

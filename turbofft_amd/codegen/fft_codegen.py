@@ -147,6 +147,15 @@ class KernelSpec:
         self.lds_elems = max([self.phys_const(self.E - 1, p) + 1 for p in self.pads] + [1])
         self.red_off_bytes = (self.lds_elems * self.lds_esize + 15) // 16 * 16
         self.lds_bytes = self.red_off_bytes + (3 * (self.threads // WAVE) * 8 if self.ft else 0)
+        # compact checksum words parked in LDS (ck = 3): W words per thread behind the reduction
+        # slots, four to an access, access g of thread tx at [g * threads + tx]
+        self.ck_lds = int(k.ck) == 3
+        self.ck_words = (self.n // 2 if self.R == "float" else self.n) if self.ck16 else 0
+        self.cw_off_bytes = (self.lds_bytes + 15) // 16 * 16
+        if self.ck_lds:
+            if self.ck_words % 4:
+                raise ValueError(f"{k}: parking the compact table in LDS needs a multiple of 4 words per thread")
+            self.lds_bytes = self.cw_off_bytes + self.ck_words * self.threads * 4
 
     # ---- address helpers (python side) ----
     @staticmethod
@@ -610,6 +619,26 @@ class KernelEmitter:
         ang = -2.0 * math.pi * k / 3.0
         return (1.0 - math.cos(ang)) / 2.0, -math.sin(ang) / 2.0
 
+    def emit_ft_table_park(self, c: Code, sim: bool):
+        """Block start, ck = 3: every thread reads its words of the compact table once and parks
+        them in its own LDS slots; it reads them back for every tile (no barrier: a thread only
+        ever touches its own slots).  Costs no register between tiles and no L2 traffic per tile."""
+        sp = self.s
+        pre = Code()
+        self.map_vars(pre, 0)
+        W = sp.ck_words
+        pre(f"unsigned cw0[{W}];")
+        for q in range(W):
+            pre(f"cw0[{q}] = CKW(ck, {sp.Tr * q}u, x);")
+        for g in range(W // 4):
+            pre(f"{{ tfft_cw4 v; v.x = cw0[{4 * g}]; v.y = cw0[{4 * g + 1}]; v.z = cw0[{4 * g + 2}]; v.w = cw0[{4 * g + 3}]; CWL_ST({sp.cw_off_bytes}, {g * sp.threads}u + tx, v); }}")
+        pre("(void)s;")
+        c("if (count > 0) {")
+        c.ind += 1
+        self.thread_block(c, sim, pre.text())
+        c.ind -= 1
+        c("}")
+
     def emit_ft_table_resident_load(self, c: Code, sim: bool):
         sp = self.s
         pre = Code()
@@ -631,6 +660,10 @@ class KernelEmitter:
         """Lane index of the per-tile table reads (kernels that do not keep the table in
         registers).  Opaque, so that the reads stay inside the tile loop."""
         if self.ft_table_resident():
+            return
+        if self.s.ck_lds:
+            c("unsigned txc = tx;")
+            c("OPAQUE(txc);")
             return
         c("unsigned xc = x;")
         c("OPAQUE(xc);")
@@ -669,6 +702,12 @@ class KernelEmitter:
             if self.ft_table_resident():
                 for q in range(W):
                     use(f"cwr[{q}]", q)
+            elif sp.ck_lds:
+                c(f"unsigned cw[{W}];")
+                for g in range(W // 4):
+                    c(f"{{ const tfft_cw4 v = CWL_LD({sp.cw_off_bytes}, {g * sp.threads}u + txc); cw[{4 * g}] = v.x; cw[{4 * g + 1}] = v.y; cw[{4 * g + 2}] = v.z; cw[{4 * g + 3}] = v.w; }}")
+                for q in range(W):
+                    use(f"cw[{q}]", q)
             else:
                 c(f"unsigned cw[{B}];")
                 for b0 in range(0, W, B):
@@ -966,6 +1005,7 @@ class KernelEmitter:
             LT = R if sp.split else T2
             c(f"std::vector<{LT}> ldsv({sp.lds_elems}); {LT}* lds = ldsv.data();")
             c(f"std::vector<TS> ts({sp.threads}); for (auto& z : ts) z = TS();")
+            c(f"std::vector<tfft_cw4> cwlv({max(1, sp.ck_words // 4 * sp.threads if sp.ck_lds else 1)}); tfft_cw4* cwl = cwlv.data(); const long long cwl_limit = (long long)cwlv.size(); (void)cwl; (void)cwl_limit;")
         else:
             wv = int(sp.key.wv)
             c(f'extern "C" __global__ __launch_bounds__({sp.threads})' + (f" __attribute__((amdgpu_waves_per_eu({wv}, {wv})))" if wv else ""))
@@ -1034,6 +1074,8 @@ class KernelEmitter:
                 c("const bool hold = count == 1 && a.ft.correct != 0;")
             if self.ft_table_resident():
                 self.emit_ft_table_resident_load(c, sim)
+            elif sp.ck_lds:
+                self.emit_ft_table_park(c, sim)
             c("for (int it = 0; it < count + extra; ++it) {")
             c.ind += 1
             c("const bool is_redo = it >= count;")

@@ -40,7 +40,8 @@ class PlanRow:
     xc: Tuple[int, ...] = ()         # optional columns 28-30: consecutive tiles per XCD (run time only; 0 = 64)
     ck: Tuple[int, ...] = ()         # optional columns 31-33: the fault-tolerant kernel of the launch reads the compact
                                      # (half-precision cotangent) form of the checksum table (fp32 only): 1 = words kept in
-                                     # registers by blocks of fewer than 1024 threads, 2 = read again for every tile
+                                     # registers by blocks of fewer than 1024 threads, 2 = read again for every tile,
+                                     # 3 = parked in LDS behind the exchange buffer (each thread its own words)
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -89,13 +90,14 @@ class KernelKey:
                      # (row1, rowT): inverse = swap . forward . swap
     ck: int = 0      # > 0: fault-tolerant fp32 kernel that reads the compact checksum table (one half-precision
                      # cotangent per element, two per 32-bit word); 1: the words stay in registers for the tiles
-                     # of a block where the block has fewer than 1024 threads, 2: they are read again for every tile
+                     # of a block where the block has fewer than 1024 threads, 2: they are read again for every tile,
+                     # 3: every thread parks its words in LDS when the block starts and reads them back per tile
 
     @property
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf == 1 else (f"_p{self.pf}" if self.pf else "")) + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2", 3: "_h3"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:

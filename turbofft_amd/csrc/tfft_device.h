@@ -107,6 +107,10 @@ __device__ __forceinline__ float tfft_ckh(unsigned w, int hi) {
 }
 #define CKH(w, hi) tfft_ckh((w), (hi))
 #define CKF(w) __uint_as_float(w)
+// a thread's compact-table words parked in LDS behind the exchange buffer, four to an access
+typedef uint4 tfft_cw4;
+#define CWL_ST(off, i, v) (((tfft_cw4*)(lds_raw + (off)))[(i)] = (v))
+#define CWL_LD(off, i) (((const tfft_cw4*)(lds_raw + (off)))[(i)])
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
 // tile-independent table reads inside the tile loop instead of hoisted into registers
 #define OPAQUE(v) asm volatile("" : "+v"(v))
@@ -162,6 +166,9 @@ static inline float tfft_ckh(unsigned w, int hi) {
 #define CKH(w, hi) tfft_ckh((w), (hi))
 static inline float tfft_ckf(unsigned w) { float f; memcpy(&f, &w, sizeof f); return f; }
 #define CKF(w) tfft_ckf(w)
+struct tfft_cw4 { unsigned x, y, z, w; };
+#define CWL_ST(off, i, v) (cwl[TFFT_CHK((i), cwl_limit, "parked checksum words")] = (v))
+#define CWL_LD(off, i) (cwl[TFFT_CHK((i), cwl_limit, "parked checksum words")])
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])
 #define LST(i, v) (lds[TFFT_CHK((i), lds_limit, "lds")] = (v))
 // cross-lane fetch in the lock-step flavour: the partner's registers as snapshotted

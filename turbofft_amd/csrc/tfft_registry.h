@@ -18,7 +18,7 @@ typedef struct tfft_kernel_entry {
     int wv;              // > 0: compiled for this many wavefronts per SIMD
     int nt;              // bit 0: non-temporal tile loads, bit 1: non-temporal tile stores, bit 2: raised wave priority for the tile loads
     int inv;             // 1: component-swapping flavour for the first / last launch of an inverse plan
-    int ck;              // 1: reads the compact (half-precision cotangent) checksum table
+    int ck;              // > 0: reads the compact (cotangent) checksum table; 1 words kept in registers, 2 read per tile, 3 parked in LDS
     int threads;         // block size
     int lds_bytes;       // dynamic LDS
 } tfft_kernel_entry;
