@@ -167,6 +167,24 @@ int turbofft_plan_tb_gap(const turbofft_plan_t* plan, int launch);
 /* Override it (tests use this to make groups reproducible). */
 int turbofft_plan_set_tb_gap(turbofft_plan_t* plan, int launch, int tb_gap);
 
+/* A checksum group is the reference's thread_bs tiles of one block (fft_codegen.py:216-218,
+ * 354-384).  Here a group longer than `tiles` tiles is walked by several blocks, `tiles` each:
+ * every block leaves its threads' running checksums in slots the plan owns and takes a ticket,
+ * and the block that takes a group's last ticket adds the parts up in order and applies the
+ * reference's rule to the whole group.  Same groups, same sums, same decisions (to rounding: the
+ * sums are added in another order); no block waits for another.  A located tile is recomputed
+ * by a second launch of the same kernel that follows at once (the tile's first store came from
+ * another block, perhaps on another XCD; the kernel boundary orders the two stores), which
+ * returns at once when nothing was located.  Default 8 tiles per block (TURBOFFT_FT_PART_LEN
+ * at plan creation overrides; 0 = one block per group, as the reference), so groups of 16 and
+ * more are shared; recompute-correcting kernels that do not prefetch only.  The slots are
+ * sized at plan creation (128 MiB, plans with thread_bs above the default only) and an
+ * execution that would need more runs one block per group.  turbofft_plan_grid keeps returning
+ * the number of groups.  Executions of one fault-tolerant plan must not overlap in time (they
+ * share the slots). */
+int turbofft_plan_set_ft_part_len(turbofft_plan_t* plan, int launch, int tiles);
+int turbofft_plan_ft_part_len(const turbofft_plan_t* plan, int launch);
+
 /* ---- fault tolerance (no counterpart API in the reference; its generator
  * bakes these into the kernel text: fft_codegen.py:412-415, 495, 714-719) ---- */
 

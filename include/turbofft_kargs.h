@@ -43,6 +43,23 @@ typedef struct tfft_ft_args {
     double inj_mag;               /* added to the real part after the input checksum       */
     double err_smoothing;         /* |delta| / (err_smoothing + |mag|) > err_threshold     */
     double err_threshold;
+    /* A checksum group walked by several blocks (parts > 1, recompute-correcting kernels): the
+       launch has groups * parts blocks, block b is part b / groups of group b % groups and walks
+       tiles [part * part_len, (part + 1) * part_len) of the group's thread_bs.  Each block leaves
+       the four running checksums of every thread in `part_sums`, takes a ticket, and the block
+       that takes the group's last one adds the parts up in order and decides.  A located tile was
+       stored by another block, perhaps on another XCD, whose write-back L2 may still hold it: it
+       is not stored again by this launch but queued in `fix_list`, and a second launch of the
+       same kernel with fix_mode = 1 (any grid) recomputes the queued tiles and empties the queue. */
+    int parts;
+    int part_len;
+    void* part_sums;              /* [((group * parts + part) * 4 + v) * threads + thread] of the
+                                     kernel's real type, v = in1, in2, out1, out2             */
+    unsigned* tickets;            /* one word per group, zero between launches              */
+    long long* fix_list;          /* tiles to recompute, one slot per group                 */
+    unsigned* fix_ctl;            /* [0] tiles queued, [1] blocks of the fix-up launch that are
+                                     done; both zero between executions                       */
+    int fix_mode;                 /* 1: this launch only recomputes the queued tiles          */
 } tfft_ft_args;
 
 typedef struct tfft_kargs {

@@ -25,7 +25,9 @@ class FtArgs(C.Structure):
                 ("flagged_cap", C.c_int), ("launch", C.c_int), ("correct", C.c_int),
                 ("inj_mode", C.c_int), ("inj_every", C.c_int), ("inj_tile", C.c_longlong),
                 ("inj_s", C.c_int), ("inj_m", C.c_int), ("inj_mag", C.c_double),
-                ("err_smoothing", C.c_double), ("err_threshold", C.c_double)]
+                ("err_smoothing", C.c_double), ("err_threshold", C.c_double),
+                ("parts", C.c_int), ("part_len", C.c_int), ("part_sums", C.c_void_p), ("tickets", C.c_void_p),
+                ("fix_list", C.c_void_p), ("fix_ctl", C.c_void_p), ("fix_mode", C.c_int)]
 
 
 class KArgs(C.Structure):
@@ -107,12 +109,14 @@ def build_sim(spec: KernelSpec):
 
 
 def run_sim(spec: KernelSpec, x_in: np.ndarray, out_elems: int, kargs: KArgs, grid: int,
-            tw: np.ndarray, twhi=None, twlo=None, ck=None):
+            tw: np.ndarray, twhi=None, twlo=None, ck=None, out=None):
     lib = build_sim(spec)
     fn = getattr(lib, spec.name + "_sim")
     ct = ctype_of(spec.T2)
     x_in = np.ascontiguousarray(x_in, dtype=ct).ravel()
-    out = np.full(out_elems, np.nan + 1j * np.nan, dtype=ct)
+    if out is None:
+        out = np.full(out_elems, np.nan + 1j * np.nan, dtype=ct)
+    assert out.size == out_elems and out.dtype == ct and out.flags.c_contiguous
     tw = np.ascontiguousarray(tw, dtype=ct)
     keep = [x_in, out, tw]
     lim = np.zeros(6, dtype=np.int64)

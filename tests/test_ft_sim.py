@@ -18,7 +18,7 @@ def rnd(shape, seed):
 
 
 def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0,
-           inj_m=0, mag=100.0, seed=0, split=0, pf=0, ft=1, ck=0):
+           inj_m=0, mag=100.0, seed=0, split=0, pf=0, ft=1, ck=0, part_len=0):
     sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, ft, split, pf, ck=ck))
     N = 1 << logNi
     bs = ntiles * BS
@@ -32,15 +32,35 @@ def run_ft(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, in
         inj_mode, inj_every, inj_tile, inj_s, inj_m, mag
     ka.ft.err_smoothing, ka.ft.err_threshold = 1000.0, 1e-3
     grid = (ntiles + thread_bs - 1) // thread_bs
+    if part_len:
+        # every group is shared by ceil(thread_bs / part_len) blocks (block b: part b / groups of group b % groups)
+        parts = -(-thread_bs // part_len)
+        sums = np.full(grid * parts * 4 * sp.threads, np.nan, dtype=np.float32 if dtype == "float2" else np.float64)
+        tickets = np.zeros(grid, dtype=np.uint32)
+        fix_list = np.full(grid, -9, dtype=np.int64)
+        fix_ctl = np.zeros(2, dtype=np.uint32)
+        ka.ft.parts, ka.ft.part_len, ka.ft.part_sums, ka.ft.tickets = parts, part_len, sums.ctypes.data, tickets.ctypes.data
+        ka.ft.fix_list, ka.ft.fix_ctl = fix_list.ctypes.data, fix_ctl.ctypes.data
+        grid *= parts
     cv = O.dft_checksum_vector(N, dtype).astype(np.complex128)
     ck = (cv.real + cv.imag) + 1j * (cv.real - cv.imag)      # device form of the table
     if sp.ck16:
         ck = O.compact_table_words(N, n, dtype).view(simlib.ctype_of(dtype))   # the compact table, as the buffer type the launcher passes
-    y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype), ck=ck).reshape(bs, N)
+    y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype), ck=ck)
+    if part_len:
+        # the fix-up launch: the same kernel recomputes the tiles the first launch queued and empties the queue
+        queued = int(fix_ctl[0])
+        ka.ft.parts, ka.ft.fix_mode = 1, 1
+        y = simlib.run_sim(sp, x, bs * N, ka, 3, simlib.twiddle_table(N, dtype), ck=ck, out=y)
+        assert not fix_ctl.any()
+        assert queued == (st.detected - st.unlocatable if correct else 0)
+    y = y.reshape(bs, N)
     # the kernels keep detections and unlocatable detections; the host derives the rest the same
     # way the library does: [0] checked, [1] detected, [2] corrected, [3] uncorrectable
     counters = [st.checked, st.detected, st.detected - st.unlocatable if correct else 0, st.unlocatable]
     fl = st.pairs()
+    if part_len:
+        assert not tickets.any()            # every group's last block leaves its ticket word at zero
     return sp, x, y, counters, fl
 
 
@@ -284,3 +304,23 @@ def test_compact_checksum_table_flavour(dtype, ck, logNi, BS, n, split):
                               O.dft_checksum_vector(1 << logNi, dtype, "compact"))
     # the table's rounding leaves a residual well under the rule the flavour is used with
     assert max(abs(d.delta) / (1000.0 + abs(d.mag)) for d in clean) < (2e-4 if dtype == "float2" else 1e-7)
+
+
+@pytest.mark.parametrize("dtype,logNi,BS,n,split,pf,ck", [("float2", 8, 4, 16, 0, 0, 0), ("double2", 10, 1, 8, 1, 0, 0),
+                                                          ("float2", 9, 2, 8, 0, 0, 1), ("float2", 10, 1, 8, 1, 0, 3),
+                                                          ("double2", 7, 8, 8, 0, 0, 2)])
+@pytest.mark.parametrize("tbs,part_len,ntiles,gap", [(8, 4, 37, 3), (5, 2, 23, 2), (32, 4, 100, 2), (6, 1, 13, 1)])
+def test_groups_shared_by_several_blocks(dtype, logNi, BS, n, split, pf, ck, tbs, part_len, ntiles, gap):
+    """A checksum group walked by several blocks (each leaves its threads' running sums in the
+    group's slots, the block with the last ticket decides): same groups, same flagged tiles, same
+    counters and the same corrected output as one block per group, on the reference cadence, on
+    clean data and with a ragged last group.  (Kernels that prefetch their next tile keep whole
+    groups: the library does not share theirs.)"""
+    for inj_mode in (1, 0):
+        one = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=inj_mode, correct=1, split=split, pf=pf, ck=ck)
+        many = run_ft(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=inj_mode, correct=1, split=split, pf=pf, ck=ck, part_len=part_len)
+        assert many[3] == one[3]                       # checked, detected, corrected, uncorrectable
+        assert sorted(many[4]) == sorted(one[4])       # flagged (launch, tile) pairs
+        assert np.array_equal(many[2], one[2])         # recomputed tiles are bit-identical
+        if inj_mode == 1:
+            assert one[3][1] > 0                        # the cadence raises detections (long groups may miss some)

@@ -574,3 +574,48 @@ def test_offline_ft_timing_runs_clean():
         ref = torch.fft.fft(x.to(torch.complex128), dim=1)
         got = out[: bs * N].view(bs, N).to(torch.complex128)
         assert (torch.linalg.vector_norm(got - ref) / torch.linalg.vector_norm(ref)).item() < (1e-5 if dt == "float2" else 1e-13) * logN
+
+
+@pytest.mark.parametrize("dt,logN,bs", [("float2", 13, 200), ("double2", 10, 333), ("float2", 16, 24), ("double2", 20, 3), ("float2", 24, 1)])
+@pytest.mark.parametrize("tbs", [12, 32])
+def test_groups_shared_by_several_blocks(dt, logN, bs, tbs):
+    """Long groups are walked by several blocks (partial checksums in slots of the plan, the block
+    with a group's last ticket decides, a second launch recomputes the located tiles): flagged
+    tiles, counters and the corrected output equal those of one block per group -- with injected
+    errors, on clean data, with ragged last groups and parts, and again on a second execution
+    (ticket words and the queue are back at zero)."""
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=tbs)
+    assert all(plan.ft_part_len(i) == (8 if tbs > 8 else 0) for i in range(plan.launches))     # the default: parts of 8 tiles
+    gaps = [7, 5, 3][:plan.launches]
+    for i, g in enumerate(gaps):
+        plan.set_tb_gap(i, g)
+    x = make(bs, 1 << logN, dt, 90 + logN)
+    row = O.PlanRow.from_list(plan.plan_row())
+    clean, _ = O.ft_plan_model(x, row, dt, tbs, gaps, None)
+    li = plan.launches - 1
+    mag = 100.0 if logN <= 10 else float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[-1])) / 0.366))
+    ntiles = O.launch_geometry(row, bs)[li].ntiles
+    every = (tbs - 1) * gaps[li] + 3
+    plan.set_ft_params(1000.0, 1e-3, correct=1)
+    res = {}
+    for mode in ("shared", "shared again", "whole"):
+        for i in range(plan.launches):
+            plan.set_ft_part_len(i, 0 if mode == "whole" else 3)                 # 3: ragged last parts as well
+        plan.set_injection(2, launch=li, every=every, tile_phase=1, s=0, m=0, mag=mag)
+        y, c = run(plan, x)
+        plan.set_injection(0)
+        y0, c0 = run(plan, x)
+        assert c0["detected"] == 0 and c0["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
+        res[mode] = (y, c, y0)
+    y, c, y0 = res["whole"]
+    injs = [O.Injection(t, 0, 0, mag) for t in range(1, ntiles, every)]
+    dec, _ = O.ft_plan_model(x, row, dt, tbs, gaps, injs, inj_launch=li)
+    model = sorted((l, d.tile) for l, dl in enumerate(dec) for d in dl if d.detected)
+    assert sorted(c["flagged"]) == model and len(model) > 0
+    for mode in ("shared", "shared again"):
+        ys, cs, ys0 = res[mode]
+        assert sorted(cs["flagged"]) == sorted(c["flagged"])
+        assert (cs["checked"], cs["detected"], cs["corrected"], cs["uncorrectable"]) == (c["checked"], c["detected"], c["corrected"], c["uncorrectable"])
+        assert np.array_equal(ys, y) and np.array_equal(ys0, y0) and np.array_equal(ys, ys0)
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    plan.close()

@@ -78,6 +78,8 @@ def lib() -> C.CDLL:
     L.turbofft_plan_kernel_name.restype = C.c_char_p
     L.turbofft_plan_tb_gap.argtypes = [vp, i]
     L.turbofft_plan_set_tb_gap.argtypes = [vp, i, i]
+    L.turbofft_plan_set_ft_part_len.argtypes = [vp, i, i]
+    L.turbofft_plan_ft_part_len.argtypes = [vp, i]
     L.turbofft_set_ft_params.argtypes = [vp, C.c_double, C.c_double, i]
     L.turbofft_set_injection.argtypes = [vp, i, i, i, ll, i, i, C.c_double]
     L.turbofft_get_ft_counters.argtypes = [vp] + [C.POINTER(C.c_ulonglong)] * 4 + [C.POINTER(ll), i, C.POINTER(i)]
@@ -263,6 +265,13 @@ class TurboFFT:
 
     def set_tb_gap(self, launch: int, gap: int):
         _check(lib().turbofft_plan_set_tb_gap(self._h, launch, gap))
+
+    def ft_part_len(self, launch: int) -> int:
+        """Tiles of a checksum group one block walks (0: the whole group)."""
+        return lib().turbofft_plan_ft_part_len(self._h, launch)
+
+    def set_ft_part_len(self, launch: int, tiles: int):
+        _check(lib().turbofft_plan_set_ft_part_len(self._h, launch, tiles))
 
     # ---- execution ----
     def exec(self, in_ptr: int, out_ptr: int, bs: int, stream: int = 0):

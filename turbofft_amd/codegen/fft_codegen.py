@@ -633,7 +633,7 @@ class KernelEmitter:
         for g in range(W // 4):
             pre(f"{{ tfft_cw4 v; v.x = cw0[{4 * g}]; v.y = cw0[{4 * g + 1}]; v.z = cw0[{4 * g + 2}]; v.w = cw0[{4 * g + 3}]; CWL_ST({sp.cw_off_bytes}, {g * sp.threads}u + tx, v); }}")
         pre("(void)s;")
-        c("if (count > 0) {")
+        c("if (it0 < it1) {")
         c.ind += 1
         self.thread_block(c, sim, pre.text())
         c.ind -= 1
@@ -650,7 +650,7 @@ class KernelEmitter:
             for e in range(sp.n):
                 pre(f"cvr[{e}] = {self.TWLU}(ck, {sp.Tr * e}u, x);")
         pre("(void)s;")
-        c("if (count > 0) {")
+        c("if (it0 < it1) {")
         c.ind += 1
         self.thread_block(c, sim, pre.text())
         c.ind -= 1
@@ -1039,20 +1039,34 @@ class KernelEmitter:
         c(f"const {T2}* twhi = (const {T2}*)a.tw_hi; const {T2}* twlo = (const {T2}*)a.tw_lo; const {T2}* ck = (const {T2}*)a.ft.cksum;")
         c("(void)twhi; (void)twlo; (void)ck;")
         # tile group of this block (fft_codegen.py:218,260-261 with a rounded-up grid)
+        parts = sp.ft and not sp.dc       # the group of a block may be shared with other blocks
+        if parts:
+            # a group walked by several blocks: block b is part b / groups of group b % groups
+            c("long long ngroups = grid; unsigned part = 0;")
+            c("if (a.ft.parts > 1) { ngroups = grid / a.ft.parts; part = (unsigned)(bx / ngroups); bx = bx % ngroups; }")
+        else:
+            c("const long long ngroups = grid;")
         c("long long gstride = 1, tile0 = bx;")
         c("int count = bx < a.ntiles ? 1 : 0;")
         c("if (a.thread_bs > 1) {")
-        c("    const unsigned ub = (unsigned)bx, gap = (unsigned)a.tb_gap, ug = (unsigned)grid, tbs = (unsigned)a.thread_bs;")
+        c("    const unsigned ub = (unsigned)bx, gap = (unsigned)a.tb_gap, ug = (unsigned)ngroups, tbs = (unsigned)a.thread_bs;")
         c("    const unsigned chunk = ub / gap;")
         c("    const unsigned gs = ((chunk + 1u) * gap <= ug) ? gap : (ug - chunk * gap);")
         c("    const unsigned long long t0 = (unsigned long long)chunk * gap * tbs + ub % gap;")
         c("    gstride = gs; tile0 = (long long)t0; count = 0;")
         c("    if (tile0 < a.ntiles) { const unsigned left = (unsigned)((a.ntiles - tile0 + gs - 1) / gs); count = left < tbs ? (int)left : (int)tbs; }")
         c("}")
+        # the tiles [it0, it1) of the group are this block's
+        c("int it0 = 0, it1 = count;")
+        if parts:
+            c("if (a.ft.parts > 1) { it0 = (int)part * a.ft.part_len; it1 = it0 + a.ft.part_len < count ? it0 + a.ft.part_len : count; if (it0 > it1) it0 = it1; }")
+            # the fix-up launch: no tiles of its own, only queued ones (block b takes entries b, b + grid, ...)
+            c("if (a.ft.fix_mode) { it0 = 0; it1 = 0; }")
+        c("const long long tile_first = tile0 + it0 * gstride; (void)tile_first;")
         if sp.pf:
-            c("if (count > 0) {")
+            c("if (it0 < it1) {")
             c.ind += 1
-            self.emit_tile_decode(c, "tile0", "_n")
+            self.emit_tile_decode(c, "tile_first", "_n")
             pre = Code()
             self.map_vars(pre, 0)
             self.emit_load(pre, "rn", "_n", elems=range(sp.pfk) if sp.pfk else None)
@@ -1062,10 +1076,12 @@ class KernelEmitter:
         if sp.ft:
             # checksum groups run: one per block, counted once per launch by its first block
             if sim:
-                c("if (pbx == 0) a.ft.counters[0] += (unsigned long long)grid;")
+                c("if (pbx == 0 && !a.ft.fix_mode) a.ft.counters[0] += (unsigned long long)ngroups;")
             else:
-                c("if (blockIdx.x == 0 && tx == 0) atomicAdd(&a.ft.counters[0], (unsigned long long)grid);")
+                c("if (blockIdx.x == 0 && tx == 0 && !a.ft.fix_mode) atomicAdd(&a.ft.counters[0], (unsigned long long)ngroups);")
             c("long long redo_tile = -1; int extra = 0;")
+            if parts:
+                c("if (a.ft.fix_mode) { const long long nfix = (long long)a.ft.fix_ctl[0]; if (pbx_raw < nfix) extra = (int)((nfix - pbx_raw + grid - 1) / grid); }")
             if sp.dc:
                 # A group of a single tile (thread_bs = 1, or a ragged last group) is verified
                 # before its result leaves the registers: nothing is stored until the block has
@@ -1076,9 +1092,11 @@ class KernelEmitter:
                 self.emit_ft_table_resident_load(c, sim)
             elif sp.ck_lds:
                 self.emit_ft_table_park(c, sim)
-            c("for (int it = 0; it < count + extra; ++it) {")
+            c("for (int it = it0; it < it1 + extra; ++it) {")
             c.ind += 1
-            c("const bool is_redo = it >= count;")
+            c("const bool is_redo = it >= it1;")
+            if parts:
+                c("if (is_redo && a.ft.fix_mode) redo_tile = a.ft.fix_list[pbx_raw + (long long)(it - it1) * grid];")
             c("const long long tile = is_redo ? redo_tile : tile0 + it * gstride;")
             c(f"const {R} cntf = ({R})(it + 1);")
             c("bool inj_hit = false;")
@@ -1086,11 +1104,11 @@ class KernelEmitter:
             c("else if (a.ft.inj_mode == 2) inj_hit = (tile % a.ft.inj_every) == a.ft.inj_tile;")
             c("(void)cntf; (void)inj_hit;")
         else:
-            c("for (int it = 0; it < count; ++it) {")
+            c("for (int it = it0; it < it1; ++it) {")
             c.ind += 1
             c("const long long tile = tile0 + it * gstride;")
         if sp.pf:
-            c("const bool has_next = it + 1 < count;")
+            c("const bool has_next = it + 1 < it1;")
             c("const long long tile_n = tile0 + (long long)(it + 1) * gstride;")
             c("(void)has_next; (void)tile_n;")
         self.emit_tile_decode(c)
@@ -1116,7 +1134,7 @@ class KernelEmitter:
                 self.thread_block(c, sim, st.text())
             if sp.pf:
                 # the tile to recompute is known only now: fetch it for the extra trip
-                c("if (extra && it == count - 1) {")
+                c("if (extra && it == it1 - 1) {")
                 c.ind += 1
                 self.emit_tile_decode(c, "redo_tile", "_n")
                 pre = Code()
@@ -1127,6 +1145,15 @@ class KernelEmitter:
                 c("}")
         c.ind -= 1
         c("}")  # tile loop
+        if parts:
+            # every block of the fix-up launch has read the queue length before it gets here
+            if sim:
+                c("if (a.ft.fix_mode && ++a.ft.fix_ctl[1] == (unsigned)grid) { a.ft.fix_ctl[0] = 0; a.ft.fix_ctl[1] = 0; }")
+            else:
+                c("if (a.ft.fix_mode) {")
+                c("    __syncthreads();")
+                c("    if (tx == 0 && atomicAdd(&a.ft.fix_ctl[1], 1u) == (unsigned)grid - 1u) { atomicExch(&a.ft.fix_ctl[0], 0u); atomicExch(&a.ft.fix_ctl[1], 0u); }")
+                c("}")
         if sim:
             c.ind -= 1
             c("}")  # block loop
@@ -1150,14 +1177,57 @@ class KernelEmitter:
         c.ind -= 1
         c("}")
 
+    def emit_ft_handoff(self, c: Code, sim: bool):
+        """A group shared by several blocks (a.ft.parts > 1), after the block's last tile: leave
+        every thread's four running checksums in the group's slots, take a ticket; the block that
+        takes the last ticket of the group adds the parts up in part order (so the sums do not
+        depend on which block comes last) and goes on to decide for the whole group, every other
+        block is done.  Nobody waits for anybody."""
+        sp = self.s
+        R = self.R
+        T = sp.threads
+        c("if (a.ft.parts > 1) {")
+        c.ind += 1
+        c(f"{R}* ps = ({R}*)a.ft.part_sums;")
+        c("const unsigned nparts = (unsigned)((count + a.ft.part_len - 1) / a.ft.part_len);      // parts of this group that hold tiles")
+        c(f"const unsigned long long slot0 = (unsigned long long)bx * (unsigned)a.ft.parts * {4 * T}ull;")
+        if sim:
+            c(f"for (unsigned tx = 0; tx < {T}u; ++tx) {{ {R}* q = ps + slot0 + (unsigned long long)part * {4 * T}ull + tx; q[0] = ts[tx].fin1; q[{T}] = ts[tx].fin2; q[{2 * T}] = ts[tx].fo1; q[{3 * T}] = ts[tx].fo2; }}")
+            c("const unsigned ticket = a.ft.tickets[bx]++;")
+            c("if (ticket != nparts - 1) break;")
+            c("a.ft.tickets[bx] = 0;")
+            c(f"for (unsigned tx = 0; tx < {T}u; ++tx) {{")
+            c("    ts[tx].fin1 = ts[tx].fin2 = ts[tx].fo1 = ts[tx].fo2 = 0;")
+            c(f"    for (unsigned pp = 0; pp < nparts; ++pp) {{ const {R}* q = ps + slot0 + (unsigned long long)pp * {4 * T}ull + tx; ts[tx].fin1 += q[0]; ts[tx].fin2 += q[{T}]; ts[tx].fo1 += q[{2 * T}]; ts[tx].fo2 += q[{3 * T}]; }}")
+            c("}")
+        else:
+            c(f"{{ {R}* q = ps + slot0 + (unsigned long long)part * {4 * T}ull + tx; tfft_ps_store(q, fin1); tfft_ps_store(q + {T}, fin2); tfft_ps_store(q + {2 * T}, fo1); tfft_ps_store(q + {3 * T}, fo2); }}")
+            c("__syncthreads();                       // every wave has waited for its stores: the sums are in memory before the ticket is taken")
+            c(f"unsigned* lastp = (unsigned*)(lds_raw + {sp.red_off_bytes});")
+            c("if (tx == 0) {")
+            c("    const unsigned ticket = atomicAdd(&a.ft.tickets[bx], 1u);")
+            c("    lastp[0] = ticket == nparts - 1 ? 1u : 0u;")
+            c("    if (ticket == nparts - 1) a.ft.tickets[bx] = 0u;      // every part has come by: ready for the next launch")
+            c("}")
+            c("__syncthreads();")
+            c("const bool last = lastp[0] != 0u;")
+            c("__syncthreads();                       // the slot is reused by the reduction below")
+            c("if (!last) break;")
+            c("fin1 = 0; fin2 = 0; fo1 = 0; fo2 = 0;      // (the other parts' sums are read after their tickets were seen)")
+            c(f"for (unsigned pp = 0; pp < nparts; ++pp) {{ const {R}* q = ps + slot0 + (unsigned long long)pp * {4 * T}ull + tx; fin1 += tfft_ps_load(q); fin2 += tfft_ps_load(q + {T}); fo1 += tfft_ps_load(q + {2 * T}); fo2 += tfft_ps_load(q + {3 * T}); }}")
+        c.ind -= 1
+        c("}")
+
     def emit_ft_decide(self, c: Code, sim: bool):
         """Block-wide reduction and the detect / locate decision
         (fft_codegen.py:432-503), then scheduling of the recompute."""
         sp = self.s
         R = self.R
         nw = sp.threads // WAVE
-        c("if (it == count - 1) {")
+        c("if (it == it1 - 1) {")
         c.ind += 1
+        if not sp.dc:
+            self.emit_ft_handoff(c, sim)
         c(f"{R} delta, mag, delta2;")
         if sim:
             c("delta = 0; mag = 0; delta2 = 0;")
@@ -1195,7 +1265,18 @@ class KernelEmitter:
             c("if (!valid) atomicAdd(sc + 1, 1ull);")
         c.ind -= 1
         c("}")
-        c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")
+        if sp.dc:
+            c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")
+        else:
+            c("if (valid && a.ft.correct) {")
+            c("    if (a.ft.parts > 1) {")
+            c("        // the tile was stored by another block: it is recomputed by the fix-up launch")
+            if sim:
+                c("        a.ft.fix_list[a.ft.fix_ctl[0]++] = bad;")
+            else:
+                c("        if (tx == 0) a.ft.fix_list[atomicAdd(&a.ft.fix_ctl[0], 1u)] = bad;")
+            c("    } else { redo_tile = bad; extra = 1; }")
+            c("}")
         c.ind -= 1
         c("}")
 

@@ -107,6 +107,12 @@ __device__ __forceinline__ float tfft_ckh(unsigned w, int hi) {
 }
 #define CKH(w, hi) tfft_ckh((w), (hi))
 #define CKF(w) __uint_as_float(w)
+// Partial checksums handed from block to block: device-scope relaxed atomic accesses, which go
+// past the XCD's own L2 to memory.  With them the hand-off needs no device-scope fence -- on this
+// part a release writes the whole L2 back and an acquire invalidates it, and thousands of blocks
+// doing that per launch made the launch four to six times slower.
+template <typename T> __device__ __forceinline__ void tfft_ps_store(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+template <typename T> __device__ __forceinline__ T tfft_ps_load(const T* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 // a thread's compact-table words parked in LDS behind the exchange buffer, four to an access
 typedef uint4 tfft_cw4;
 #define CWL_ST(off, i, v) (((tfft_cw4*)(lds_raw + (off)))[(i)] = (v))
@@ -167,6 +173,8 @@ static inline float tfft_ckh(unsigned w, int hi) {
 static inline float tfft_ckf(unsigned w) { float f; memcpy(&f, &w, sizeof f); return f; }
 #define CKF(w) tfft_ckf(w)
 struct tfft_cw4 { unsigned x, y, z, w; };
+template <typename T> static inline void tfft_ps_store(T* p, T v) { *p = v; }
+template <typename T> static inline T tfft_ps_load(const T* p) { return *p; }
 #define CWL_ST(off, i, v) (cwl[TFFT_CHK((i), cwl_limit, "parked checksum words")] = (v))
 #define CWL_LD(off, i) (cwl[TFFT_CHK((i), cwl_limit, "parked checksum words")])
 #define LLD(i) (lds[TFFT_CHK((i), lds_limit, "lds")])

@@ -61,6 +61,12 @@ namespace {
     } while (0)
 
 constexpr double kPi = 3.14159265358979323846;
+// checksum groups shared by several blocks: tiles a block walks, bytes of partial-sum slots and
+// ticket words a fault-tolerant plan with longer groups holds
+constexpr int kPartLen = 8;
+constexpr size_t kPartSumsBytes = (size_t)128 << 20;
+constexpr long long kPartTickets = 1ll << 20;
+constexpr long long kFixGrid = 256;         // blocks of the launch that recomputes queued tiles
 // smallest err_threshold the compact checksum tables serve: half-precision entries (fp32 kernels)
 // leave up to 1e-4 of the checksum magnitude as residual on clean data, single-precision ones
 // (fp64 kernels) 1e-8
@@ -214,6 +220,16 @@ struct turbofft_plan {
     unsigned long long* counters = nullptr;   // 8 x u64
     long long* flagged = nullptr;
     int flagged_cap = 4096;
+    // Checksum groups shared by several blocks (plans whose groups are longer than ft_part_len
+    // tiles): slots for the blocks' partial checksums and one ticket word per group, sized once
+    // at plan creation; an execution that would need more walks whole groups per block.
+    int ft_part_len[3] = {0, 0, 0};           // tiles per block (0: the whole group)
+    void* part_sums = nullptr;
+    unsigned* tickets = nullptr;
+    long long* fix_list = nullptr;            // tiles_n slots: tiles the fix-up launch recomputes
+    unsigned* fix_ctl = nullptr;              // queue length, finished blocks of the fix-up launch
+    size_t part_sums_bytes = 0;
+    long long tickets_n = 0;
     // FT run-time parameters
     double err_smoothing = 1000.0, err_threshold = 1e-3;
     int correct = 0;
@@ -303,6 +319,10 @@ void turbofft_plan_destroy(turbofft_plan_t* p) {
     }
     if (p->counters) (void)hipFree(p->counters);
     if (p->flagged) (void)hipFree(p->flagged);
+    if (p->part_sums) (void)hipFree(p->part_sums);
+    if (p->tickets) (void)hipFree(p->tickets);
+    if (p->fix_list) (void)hipFree(p->fix_list);
+    if (p->fix_ctl) (void)hipFree(p->fix_ctl);
     delete p;
 }
 
@@ -530,6 +550,22 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         HIP_TRY(hipMemset(p->counters, 0, TFFT_FT_COUNTER_WORDS * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void**)&p->flagged, sizeof(long long) * 2 * p->flagged_cap));
         HIP_TRY(hipMemset(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap));
+        // Long groups are walked by several blocks, kPartLen tiles each (TURBOFFT_FT_PART_LEN
+        // overrides, 0 switches it off): a block that walks many tiles in sequence gives up the
+        // overlap that block scheduling provides, and few long groups leave CUs idle.
+        int part_len = kPartLen;
+        if (const char* e = getenv("TURBOFFT_FT_PART_LEN")) part_len = atoi(e);
+        if (part_len > 0 && p->thread_bs > part_len) {
+            for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = part_len;
+            p->part_sums_bytes = kPartSumsBytes;
+            p->tickets_n = kPartTickets;
+            HIP_TRY(hipMalloc(&p->part_sums, p->part_sums_bytes));
+            HIP_TRY(hipMalloc((void**)&p->tickets, sizeof(unsigned) * (size_t)p->tickets_n));
+            HIP_TRY(hipMemset(p->tickets, 0, sizeof(unsigned) * (size_t)p->tickets_n));
+            HIP_TRY(hipMalloc((void**)&p->fix_list, sizeof(long long) * (size_t)p->tickets_n));
+            HIP_TRY(hipMalloc((void**)&p->fix_ctl, 2 * sizeof(unsigned)));
+            HIP_TRY(hipMemset(p->fix_ctl, 0, 2 * sizeof(unsigned)));
+        }
     }
     return TURBOFFT_OK;
 }
@@ -610,6 +646,19 @@ int turbofft_plan_set_tb_gap(turbofft_plan_t* p, int launch, int tb_gap) {
     return TURBOFFT_OK;
 }
 
+int turbofft_plan_set_ft_part_len(turbofft_plan_t* p, int launch, int tiles) {
+    if (!p || launch < 0 || launch >= p->launches || tiles < 0) return fail(TURBOFFT_EINVAL, "bad argument");
+    if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
+    if (tiles > 0 && !p->part_sums) return fail(TURBOFFT_EINVAL, "the plan holds no slots for shared groups (thread_bs %d)", p->thread_bs);
+    p->ft_part_len[launch] = tiles;
+    return TURBOFFT_OK;
+}
+
+int turbofft_plan_ft_part_len(const turbofft_plan_t* p, int launch) {
+    if (!p || launch < 0 || launch >= p->launches) return 0;
+    return p->ft_part_len[launch];
+}
+
 int turbofft_set_ft_params(turbofft_plan_t* p, double err_smoothing, double err_threshold, int correct) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
@@ -665,6 +714,8 @@ int turbofft_reset_ft_counters(turbofft_plan_t* p) {
     if (rc) return rc;
     HIP_TRY(hipMemsetAsync(p->counters, 0, TFFT_FT_COUNTER_WORDS * sizeof(unsigned long long), st));
     HIP_TRY(hipMemsetAsync(p->flagged, 0xff, sizeof(long long) * 2 * p->flagged_cap, st));
+    if (p->tickets) HIP_TRY(hipMemsetAsync(p->tickets, 0, sizeof(unsigned) * (size_t)p->tickets_n, st));
+    if (p->fix_ctl) HIP_TRY(hipMemsetAsync(p->fix_ctl, 0, 2 * sizeof(unsigned), st));
     HIP_TRY(hipStreamSynchronize(st));
     return TURBOFFT_OK;
 }
@@ -916,6 +967,22 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         }
         long long grid = (a.ntiles + a.thread_bs - 1) / a.thread_bs;
         if (grid < 1) continue;
+        long long fix_grid = 0;
+        if (p->if_ft && k->ft == 1 && !k->pf && p->ft_part_len[i] > 0 && a.thread_bs > p->ft_part_len[i]) {
+            // groups longer than ft_part_len tiles: several blocks per group, where the plan's slots suffice
+            const long long parts = (a.thread_bs + p->ft_part_len[i] - 1) / p->ft_part_len[i];
+            const unsigned long long need = (unsigned long long)grid * parts * 4ull * k->threads * (p->esize / 2);
+            if (need <= p->part_sums_bytes && grid <= p->tickets_n && grid * parts <= 0x7fffffffll) {
+                a.ft.parts = (int)parts;
+                a.ft.part_len = p->ft_part_len[i];
+                a.ft.part_sums = p->part_sums;
+                a.ft.tickets = p->tickets;
+                a.ft.fix_list = p->fix_list;
+                a.ft.fix_ctl = p->fix_ctl;
+                if (a.ft.correct) fix_grid = grid < kFixGrid ? grid : kFixGrid;
+                grid *= parts;
+            }
+        }
         if (grid > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "grid of %lld blocks exceeds the launch limit", grid);
         const void* in_arg = src[i];
         void* out_arg = dst[i];
@@ -924,6 +991,15 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         if (o.ev) HIP_TRY(hipEventRecord(o.ev[i], (hipStream_t)stream));
         HIP_TRY(hipLaunchKernel(k->func, dim3((unsigned)grid), dim3((unsigned)k->threads), args, (size_t)k->lds_bytes,
                                 (hipStream_t)stream));
+        if (fix_grid) {
+            // groups shared by several blocks: tiles found wrong are recomputed by a second launch of
+            // the same kernel (a kernel boundary orders the two stores of such a tile, which come
+            // from blocks on different XCDs); with nothing queued its blocks return at once
+            a.ft.parts = 1;
+            a.ft.fix_mode = 1;
+            HIP_TRY(hipLaunchKernel(k->func, dim3((unsigned)fix_grid), dim3((unsigned)k->threads), args, (size_t)k->lds_bytes,
+                                    (hipStream_t)stream));
+        }
         if (o.sync_each) HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     }
     if (o.ev) HIP_TRY(hipEventRecord(o.ev[p->launches], (hipStream_t)stream));
