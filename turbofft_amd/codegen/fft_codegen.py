@@ -1043,7 +1043,10 @@ class KernelEmitter:
         if parts:
             # a group walked by several blocks: block b is part b / groups of group b % groups
             c("long long ngroups = grid; unsigned part = 0;")
-            c("if (a.ft.parts > 1) { ngroups = grid / a.ft.parts; part = (unsigned)(bx / ngroups); bx = bx % ngroups; }")
+            c("if (a.ft.parts > 1) {")
+            c("    const unsigned ng = (unsigned)grid / (unsigned)a.ft.parts, ub = (unsigned)bx;")
+            c("    ngroups = ng; part = tfft_uni(ub / ng); bx = (long long)tfft_uni(ub % ng);")
+            c("}")
         else:
             c("const long long ngroups = grid;")
         c("long long gstride = 1, tile0 = bx;")
@@ -1057,6 +1060,8 @@ class KernelEmitter:
         c("    if (tile0 < a.ntiles) { const unsigned left = (unsigned)((a.ntiles - tile0 + gs - 1) / gs); count = left < tbs ? (int)left : (int)tbs; }")
         c("}")
         # the tiles [it0, it1) of the group are this block's
+        if parts:
+            c("gstride = tfft_uni(gstride); tile0 = tfft_uni(tile0); count = tfft_uni(count);")
         c("int it0 = 0, it1 = count;")
         if parts:
             c("if (a.ft.parts > 1) { it0 = (int)part * a.ft.part_len; it1 = it0 + a.ft.part_len < count ? it0 + a.ft.part_len : count; if (it0 > it1) it0 = it1; }")
@@ -1146,6 +1151,7 @@ class KernelEmitter:
         c.ind -= 1
         c("}")  # tile loop
         if parts:
+            self.emit_ft_decide(c, sim, shared=True)
             # every block of the fix-up launch has read the queue length before it gets here
             if sim:
                 c("if (a.ft.fix_mode && ++a.ft.fix_ctl[1] == (unsigned)grid) { a.ft.fix_ctl[0] = 0; a.ft.fix_ctl[1] = 0; }")
@@ -1218,16 +1224,27 @@ class KernelEmitter:
         c.ind -= 1
         c("}")
 
-    def emit_ft_decide(self, c: Code, sim: bool):
+    def emit_ft_decide(self, c: Code, sim: bool, shared: bool = False):
         """Block-wide reduction and the detect / locate decision
-        (fft_codegen.py:432-503), then scheduling of the recompute."""
+        (fft_codegen.py:432-503), then scheduling of the recompute.  Emitted inside the tile loop
+        after the group's last tile (a located tile is recomputed by one more trip through the
+        loop) and, `shared`, once more behind the loop for a group that several blocks walked:
+        there the block first hands its sums on, only the block with the group's last ticket
+        decides, and a located tile is queued for the fix-up launch.  (With the hand-off inside
+        the loop the loop body needed about nine more vector registers.)"""
         sp = self.s
         R = self.R
         nw = sp.threads // WAVE
-        c("if (it == it1 - 1) {")
-        c.ind += 1
-        if not sp.dc:
+        if shared:
+            c("if (a.ft.parts > 1 && it0 < it1) do {")
+            c.ind += 1
             self.emit_ft_handoff(c, sim)
+        elif sp.dc:
+            c("if (it == it1 - 1) {")
+            c.ind += 1
+        else:
+            c("if (it == it1 - 1 && a.ft.parts <= 1) {")
+            c.ind += 1
         c(f"{R} delta, mag, delta2;")
         if sim:
             c("delta = 0; mag = 0; delta2 = 0;")
@@ -1265,20 +1282,18 @@ class KernelEmitter:
             c("if (!valid) atomicAdd(sc + 1, 1ull);")
         c.ind -= 1
         c("}")
-        if sp.dc:
-            c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")
-        else:
-            c("if (valid && a.ft.correct) {")
-            c("    if (a.ft.parts > 1) {")
-            c("        // the tile was stored by another block: it is recomputed by the fix-up launch")
+        if shared:
+            # the tile was stored by another block, perhaps on another XCD: the fix-up launch recomputes it
             if sim:
-                c("        a.ft.fix_list[a.ft.fix_ctl[0]++] = bad;")
+                c("if (valid && a.ft.correct) a.ft.fix_list[a.ft.fix_ctl[0]++] = bad;")
             else:
-                c("        if (tx == 0) a.ft.fix_list[atomicAdd(&a.ft.fix_ctl[0], 1u)] = bad;")
-            c("    } else { redo_tile = bad; extra = 1; }")
+                c("if (valid && a.ft.correct && tx == 0) a.ft.fix_list[atomicAdd(&a.ft.fix_ctl[0], 1u)] = bad;")
+            c.ind -= 1
+            c("} while (0);")
+        else:
+            c("if (valid && a.ft.correct) { redo_tile = bad; extra = 1; }")
+            c.ind -= 1
             c("}")
-        c.ind -= 1
-        c("}")
 
 
 FILE_HEADER = """// GENERATED by turbofft_amd/codegen/fft_codegen.py -- do not edit.

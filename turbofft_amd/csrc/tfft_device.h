@@ -120,6 +120,14 @@ typedef uint4 tfft_cw4;
 // makes a per-lane value opaque to the optimiser (no code is emitted): used to keep
 // tile-independent table reads inside the tile loop instead of hoisted into registers
 #define OPAQUE(v) asm volatile("" : "+v"(v))
+// a block-uniform value back into a scalar register (the integer divisions of the tile-group
+// formula run on the vector unit and leave their results, and everything derived, in VGPRs)
+__device__ __forceinline__ unsigned tfft_uni(unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ int tfft_uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ long long tfft_uni(long long v) {
+    const unsigned lo = tfft_uni((unsigned)v), hi = tfft_uni((unsigned)((unsigned long long)v >> 32));
+    return (long long)(((unsigned long long)hi << 32) | lo);
+}
 // instruction-scheduling fence: nothing may be moved across it
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 #else
@@ -157,6 +165,7 @@ extern long long tfft_sim_errors;
 #define TWLD(p, i) ((p)[TFFT_CHK((i), p##_limit, #p)])
 #define TWLDU(p, c, i) ((p)[TFFT_CHK((long long)(c) + (long long)(i), p##_limit, #p)])
 #define OPAQUE(v)
+template <typename T> static inline T tfft_uni(T v) { return v; }
 #define SCHED_FENCE()
 // compact checksum table (ck_limit counts complex elements of the buffer the launcher passed)
 #define CKW(p, c, i) (((const unsigned*)(p))[TFFT_CHK((long long)(c) + (long long)(i), (long long)(sizeof(*(p)) / 4) * ck_limit, "compact checksum table")])
