@@ -702,12 +702,19 @@ def test_seeded_random_shapes():
         plan.close()
 
 
-@pytest.mark.parametrize("dt,logN,bs,ft", [("float2", 10, 7, 0), ("double2", 16, 3, 0), ("float2", 24, 1, 0), ("float2", 12, 9, 1)])
+@pytest.mark.parametrize("dt,logN,bs,ft", [("float2", 10, 7, 0), ("double2", 16, 3, 0), ("float2", 24, 1, 0), ("float2", 12, 9, 1),
+                                           ("double2", 10, 200, 16), ("float2", 17, 20, 32)])
 def test_exec_inside_a_hip_graph(dt, logN, bs, ft):
     """turbofft_exec allocates nothing and records no memset, so a plan can be captured into
     a HIP graph; every replay (with new input written in between) must equal the eager result."""
     torch = _torch()
-    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=ft, thread_bs=2 if ft else 1)
+    # ft > 1: checksum groups of that many tiles, shared by several blocks, with injected errors
+    # that the follow-up launch corrects -- all of it inside the graph
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=ft, thread_bs=ft if ft > 1 else (2 if ft else 1))
+    if ft > 1:
+        assert plan.ft_part_len(plan.launches - 1) == 8
+        plan.set_ft_params(1000.0, 1e-3, correct=1)
+        plan.set_injection(2, every=3 * ft * plan.tb_gap(plan.launches - 1) + 1, tile_phase=1, s=0, m=0, mag=1.0e7)
     cdt = torch.complex64 if dt == "float2" else torch.complex128
     x = torch.from_numpy(make(bs, 1 << logN, dt, 50)).cuda()
     out = torch.empty(plan.out_elems(bs), dtype=cdt, device="cuda")
@@ -734,5 +741,9 @@ def test_exec_inside_a_hip_graph(dt, logN, bs, ft):
         # the groups-checked counter lives on the device: replays count like eager executions
         # (1 warm-up + 3 replays + 3 eager runs; the capture itself executes nothing)
         c = plan.ft_counters()
-        assert c["checked"] == 7 * sum(plan.grid(i, bs) for i in range(plan.launches)) and c["detected"] == 0
+        assert c["checked"] == 7 * sum(plan.grid(i, bs) for i in range(plan.launches))
+        if ft > 1:
+            assert c["detected"] > 0 and c["detected"] % 7 == 0 and c["corrected"] == c["detected"] and c["uncorrectable"] == 0
+        else:
+            assert c["detected"] == 0
     plan.close()
