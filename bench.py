@@ -17,7 +17,8 @@ whole batch.  Prints ONE JSON line:
                  (plain, checksummed, plain, ...) so that both see the same device state;
                  the ratio of the two medians (--no_ft_overhead skips it);
                  "offline" inside it is the same comparison for separate checksum passes
-                 before and after the plain plan (the reference's cufft_ft.h baseline)
+                 before and after the plain plan (the reference's cufft_ft.h baseline),
+                 "groups_of_32" the same with the reference's published group size
   prewarm_s    : untimed executions before the warm-up steps, by time rather than by count:
                  a device that has been idle clocks up over its first tenths of a second
   vendor_baseline : hipFFT (rocFFT) on the same buffers and workload, after the timed
@@ -341,6 +342,10 @@ def main():
         # the second half of the headline metric: the same workload with the fused checksums
         # (4 tiles per checksum group, no error injected), outside the timed region above
         ft_line = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param)
+        # the same with the group size of the reference's published runs (compile.sh:13): 32 tiles,
+        # which this library walks with several blocks per group
+        g32 = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param, thread_bs=32, rounds=4)
+        ft_line["groups_of_32"] = {"overhead_pct": g32["overhead_pct"], "ms_per_step": g32["ms_per_step"], "order": g32["order"]}
         # the offline scheme on the same workload: checksum pass, plain plan, checksum pass, compare
         try:
             oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 10),

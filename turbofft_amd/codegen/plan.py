@@ -42,6 +42,8 @@ class PlanRow:
                                      # (half-precision cotangent) form of the checksum table (fp32 only): 1 = words kept in
                                      # registers by blocks of fewer than 1024 threads, 2 = read again for every tile,
                                      # 3 = parked in LDS behind the exchange buffer (each thread its own words)
+    gp: Tuple[int, ...] = ()         # optional columns 34-36 (fault-tolerant tables, run time only): tiles a block walks of a
+                                     # checksum group that is shared by several blocks (0 = the library's default)
 
     @staticmethod
     def from_list(row: Sequence[int]) -> "PlanRow":
@@ -57,7 +59,7 @@ class PlanRow:
         p = PlanRow(row[0], L, tuple(row[2:2 + L]), tuple(row[5:5 + L]), tuple(row[8:8 + L]), tuple(ext[:L]),
                     tuple(ext2[:L]), tuple(ext3[:L]), row[20] if len(row) > 20 else 0,
                     tuple((row[21:24] + [0, 0, 0])[:L]), tuple((row[24:27] + [0, 0, 0])[:L]), tuple((row[27:30] + [0, 0, 0])[:L]),
-                    tuple((row[30:33] + [0, 0, 0])[:L]))
+                    tuple((row[30:33] + [0, 0, 0])[:L]), tuple((row[33:36] + [0, 0, 0])[:L]))
         if any(t not in range(8) for t in p.nt):
             raise ValueError(f"tile access policy columns must be 0..7 in row {row}")
         if L and sum(p.logNi) != p.logN:
@@ -107,7 +109,7 @@ def load_plan_csv(path: str) -> List[PlanRow]:
             line = line.strip()
             if not line or line.startswith("#"):
                 continue
-            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:33] if t.strip()]))
+            rows.append(PlanRow.from_list([int(t) for t in line.split(",")[:36] if t.strip()]))
     return rows
 
 

@@ -74,13 +74,16 @@ constexpr double kCompactMinThreshold32 = 5e-4, kCompactMinThreshold64 = 1e-6;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[33];           // 11 reference columns + optional per-launch flags: split exchange,
+    int v[36];           // 11 reference columns + optional per-launch flags: split exchange,
                          // prefetch, cross-lane last pass; then the tiles-per-block hint, the
                          // per-launch wavefronts-per-SIMD the plain kernel was compiled for and
                          // the per-launch non-temporal access bits, then the per-launch
                          // number of consecutive tiles an XCD works on (0 = 64), then the per-launch
-                         // compact-checksum-table flag of the fault-tolerant fp32 kernel
+                         // compact-checksum-table flag of the fault-tolerant kernel, then the per-launch
+                         // number of tiles a block walks of a checksum group that several blocks share
+                         // (0 = the library's default)
     int ck(int i) const { return v[30 + i]; }
+    int gp(int i) const { return v[33 + i]; }
     int nt(int i) const { return v[24 + i]; }
     int xc(int i) const { return v[27 + i]; }
     int tiles() const { return v[20]; }
@@ -106,7 +109,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 33 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 36 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -556,7 +559,8 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         int part_len = kPartLen;
         if (const char* e = getenv("TURBOFFT_FT_PART_LEN")) part_len = atoi(e);
         if (part_len > 0 && p->thread_bs > part_len) {
-            for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = part_len;
+            // (a plan row may name its own length per launch, columns 34-36 of the fault-tolerant table)
+            for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = (p->row.gp(i) > 0 && !getenv("TURBOFFT_FT_PART_LEN")) ? p->row.gp(i) : part_len;
             p->part_sums_bytes = kPartSumsBytes;
             p->tickets_n = kPartTickets;
             HIP_TRY(hipMalloc(&p->part_sums, p->part_sums_bytes));
