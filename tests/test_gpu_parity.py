@@ -288,9 +288,9 @@ def test_agrees_with_the_vendor_library(dt, logN, bs):
     plan.close()
 
 
-@pytest.mark.parametrize("dt,logN", [("float2", 26), ("float2", 29), ("double2", 27), ("double2", 29)])
-def test_plans_beyond_2p25(dt, logN):
-    # rows 26-29 (the reference's fp64 table lists them, param/A100/param_double2.csv:27-30; its
+@pytest.mark.parametrize("dt,logN", [(dt, logN) for dt in ("float2", "double2") for logN in range(25, 30)])
+def test_plans_of_2p25_and_beyond(dt, logN):
+    # row 25, the largest the reference dispatches, and rows 26-29 (the reference's fp64 table lists them, param/A100/param_double2.csv:27-30; its
     # dispatch stops at 2^25): one transform, checked with closed forms that need no second
     # transform of that size -- a unit impulse at m gives W_N^(m k), the constant gives N at k = 0 --
     # plus linearity on random data against the vendor library where that is available.
