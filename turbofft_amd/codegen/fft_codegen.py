@@ -269,6 +269,16 @@ class KernelEmitter:
             return expr
         return f"(({expr}) + ((({expr}) >> {ps}) << {pl}))"
 
+    def lds_index_at(self, base: str, base_phys: str, off: int, pad: Tuple[int, int]) -> str:
+        """Padded index of base + off, where base_phys names the padded index of base.  An offset
+        that is a multiple of the padding period moves the padded index by a constant (the shift
+        drops none of its bits), which the compiler cannot see for itself in a 1024-thread block
+        and otherwise recomputes per element (four integer instructions per LDS access)."""
+        ps, pl = pad
+        if ps < 0 or off % (1 << ps):
+            return self.lds_index(f"{base} + {off}u", pad)
+        return f"({base_phys} + {off + ((off >> ps) << pl)}u)"
+
     # ---------- radix-R DIF in registers ----------
     def emit_radix(self, c: Code, regs: Sequence[int]):
         R = len(regs)
@@ -393,9 +403,11 @@ class KernelEmitter:
             else:
                 c(f"const unsigned a0 = s + (pos0 << {ilog2(sp.BS)});")
                 step = P * sp.BS
+            if pad[0] >= 0:
+                c(f"const unsigned a0p = {self.lds_index('a0', pad)};")
             for o in range(R):
                 reg = u + U * bitrev(o, lR)
-                c(f"LST({self.lds_index(f'a0 + {step * o}u', pad)}, r[{reg}]{part});")
+                c(f"LST({self.lds_index_at('a0', 'a0p', step * o, pad)}, r[{reg}]{part});")
             c.ind -= 1
             c("}")
 
@@ -408,8 +420,10 @@ class KernelEmitter:
         else:
             c("const unsigned b0 = tx;")
             step = sp.threads
+        if pad[0] >= 0:
+            c(f"const unsigned b0p = {self.lds_index('b0', pad)};")
         for e in range(sp.n):
-            c(f"r[{e}]{part} = LLD({self.lds_index(f'b0 + {step * e}u', pad)});")
+            c(f"r[{e}]{part} = LLD({self.lds_index_at('b0', 'b0p', step * e, pad)});")
 
     # ---------- global addressing ----------
     def emit_tile_decode(self, c: Code, tile: str = "tile", sfx: str = ""):
