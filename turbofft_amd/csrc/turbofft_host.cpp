@@ -52,12 +52,17 @@ void tfft_set_error(const char* fmt, ...) {
 
 namespace {
 
+// A failed call is reported once, through the return code: the runtime's own record of it is
+// cleared, or the caller's next check of hipGetLastError() (PyTorch makes one after every launch)
+// would report this library's error as its own.
 #define HIP_TRY(expr)                                                                         \
     do {                                                                                      \
         hipError_t e_ = (expr);                                                               \
-        if (e_ != hipSuccess)                                                                 \
+        if (e_ != hipSuccess) {                                                               \
+            (void)hipGetLastError();                                                          \
             return fail(TURBOFFT_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
                         __FILE__, __LINE__);                                                  \
+        }                                                                                     \
     } while (0)
 
 constexpr double kPi = 3.14159265358979323846;
@@ -66,6 +71,7 @@ constexpr double kPi = 3.14159265358979323846;
 constexpr int kPartLen = 8;
 constexpr size_t kPartSumsBytes = (size_t)128 << 20;
 constexpr long long kPartTickets = 1ll << 20;
+constexpr int kCuLdsBytes = 160 * 1024;     // LDS of one gfx950 compute unit
 constexpr long long kFixGrid = 256;         // blocks of the launch that recomputes queued tiles
 // smallest err_threshold the compact checksum tables serve: half-precision entries (fp32 kernels)
 // leave up to 1e-4 of the checksum magnitude as residual on clean data, single-precision ones
@@ -425,6 +431,16 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     return TURBOFFT_OK;
 }
 
+// A kernel whose dynamic LDS exceeds the default per-block limit has to be opted in; one that
+// exceeds what a CU holds is refused here, before the runtime is asked.
+static int allow_lds(const tfft_kernel_entry* k, const hipDeviceProp_t& prop) {
+    if (k->lds_bytes > kCuLdsBytes)
+        return fail(TURBOFFT_ENOPLAN, "kernel %s needs %d B of LDS, a gfx950 CU has %d", k->name, k->lds_bytes, kCuLdsBytes);
+    if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
+        HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
+    return TURBOFFT_OK;
+}
+
 static int plan_build_row(turbofft_plan* p, const Row& row) {
     p->row = row;
     const Row& r = p->row;
@@ -460,15 +476,14 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
             // flavour stays available for the table modes and thresholds the compact form cannot serve
             const tfft_kernel_entry* kc = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 1, r.split(i) ? 1 : 0, 0, 0, r.wv(i), r.nt(i) & 3, 0, r.ck(i));
             if (!kc) return fail(TURBOFFT_ENOPLAN, "no compiled compact-checksum kernel for launch %d of logN=%d", i, p->logN);
-            if ((size_t)kc->lds_bytes > (size_t)prop.sharedMemPerBlock)
-                HIP_TRY(hipFuncSetAttribute(kc->func, hipFuncAttributeMaxDynamicSharedMemorySize, kc->lds_bytes));
+            if (int rc = allow_lds(kc, prop)) return rc;
             k = kc;
         }
         p->k[i] = k;
         if (p->if_ft) {
             p->k_dc[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 2, r.split(i) ? 1 : 0, 0, 0, 0, r.nt(i) & 3);
-            if (p->k_dc[i] && (size_t)p->k_dc[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
-                HIP_TRY(hipFuncSetAttribute(p->k_dc[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_dc[i]->lds_bytes));
+            if (p->k_dc[i] && p->k_dc[i]->lds_bytes > kCuLdsBytes) p->k_dc[i] = nullptr;   // no such flavour on this device
+            if (p->k_dc[i]) if (int rc = allow_lds(p->k_dc[i], prop)) return rc;
         }
         if (r.xc(i) > 0) p->xcd_chunk_l[i] = r.xc(i);
         // Inverse plans run the same launches with a component-swapping flavour of the first and
@@ -478,15 +493,12 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         if (!p->if_ft && (i == 0 || i == p->launches - 1)) {
             p->k_inv[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 0, r.split(i) ? 1 : 0, r.pf(i) > 1 ? 0 : r.pf(i),
                                       r.xl(i) ? 1 : 0, r.wv(i), r.nt(i), 1);
-            if (p->k_inv[i] && (size_t)p->k_inv[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
-                HIP_TRY(hipFuncSetAttribute(p->k_inv[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_inv[i]->lds_bytes));
+            if (p->k_inv[i]) if (int rc = allow_lds(p->k_inv[i], prop)) return rc;
         } else if (p->if_ft) {
             p->k_inv[i] = nullptr;
         }
-        if ((size_t)k->lds_bytes > (size_t)prop.sharedMemPerBlock)
-            HIP_TRY(hipFuncSetAttribute(k->func, hipFuncAttributeMaxDynamicSharedMemorySize, k->lds_bytes));
-        if (p->k_full[i] != k && (size_t)p->k_full[i]->lds_bytes > (size_t)prop.sharedMemPerBlock)
-            HIP_TRY(hipFuncSetAttribute(p->k_full[i]->func, hipFuncAttributeMaxDynamicSharedMemorySize, p->k_full[i]->lds_bytes));
+        if (int rc = allow_lds(k, prop)) return rc;
+        if (p->k_full[i] != k) if (int rc = allow_lds(p->k_full[i], prop)) return rc;
         int nb = 0;
         HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k->func, k->threads, k->lds_bytes));
         if (nb < 1) return fail(TURBOFFT_ENOPLAN, "kernel %s does not fit on a CU (LDS %d B)", k->name, k->lds_bytes);
@@ -1060,7 +1072,7 @@ struct HostPipe {
     std::vector<hipStream_t> st;
     EventSet ev;
     int alloc(void** q, size_t bytes) {
-        if (hipMalloc(q, bytes) != hipSuccess) return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes);
+        if (hipMalloc(q, bytes) != hipSuccess) { (void)hipGetLastError(); return fail(TURBOFFT_ENOMEM, "hipMalloc(%zu) failed", bytes); }
         dev.push_back(*q);
         return TURBOFFT_OK;
     }
