@@ -571,7 +571,8 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         int part_len = kPartLen;
         if (const char* e = getenv("TURBOFFT_FT_PART_LEN")) part_len = atoi(e);
         if (part_len > 0 && p->thread_bs > part_len) {
-            // (a plan row may name its own length per launch, columns 34-36 of the fault-tolerant table)
+            // (a plan row may name its own length per launch, columns 34-36 of the fault-tolerant table; groups of up to
+            // kPartLen tiles are never shared, whatever the row says: sharing them measured slower at most sizes)
             for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = (p->row.gp(i) > 0 && !getenv("TURBOFFT_FT_PART_LEN")) ? p->row.gp(i) : part_len;
             p->part_sums_bytes = kPartSumsBytes;
             p->tickets_n = kPartTickets;
