@@ -346,7 +346,8 @@ def test_detect_only_leaves_error_in_place():
     y, c = run(plan, x)
     assert c["detected"] == 1 and c["corrected"] == 0 and c["flagged"] == [(0, 5)]
     err = np.abs(y - O.fft_ref(x))
-    assert np.allclose(err[5], 100.0, rtol=1e-9) and np.delete(err, 5, axis=0).max() < 1e-9
+    hit = 5 * plan.BS[0]                      # sub-FFT 0 of tile 5 (a tile holds BS transforms)
+    assert np.allclose(err[hit], 100.0, rtol=1e-9) and np.delete(err, hit, axis=0).max() < 1e-9
 
 
 def test_threshold_rule():
@@ -593,7 +594,8 @@ def test_groups_shared_by_several_blocks(dt, logN, bs, tbs):
     row = O.PlanRow.from_list(plan.plan_row())
     clean, _ = O.ft_plan_model(x, row, dt, tbs, gaps, None)
     li = plan.launches - 1
-    mag = 100.0 if logN <= 10 else float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[-1])) / 0.366))
+    # large enough to pass the threshold whatever the group's magnitude (it grows with the tile's columns)
+    mag = max(100.0, float(np.ceil(30e-3 * (1000.0 + max(d.mag for d in clean[-1])) / 0.366)))
     ntiles = O.launch_geometry(row, bs)[li].ntiles
     every = (tbs - 1) * gaps[li] + 3
     plan.set_ft_params(1000.0, 1e-3, correct=1)
