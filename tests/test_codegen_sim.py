@@ -224,3 +224,20 @@ def test_inverse_flavour_of_a_single_launch_kernel(dtype, logNi, BS, n, xl):
     y = simlib.run_sim(sp, x, bs * N, ka, ka.ntiles, simlib.twiddle_table(N, dtype)).reshape(bs, N)
     ref = np.fft.ifft(x.astype(simlib.ctype_of(dtype)).astype(np.complex128), axis=1) * N
     assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)
+
+
+@pytest.mark.parametrize("pad", [(5, 0), (4, 1), (6, 2), (3, 0), (-1, 0)])
+def test_padded_lds_index_of_base_plus_offset(pad):
+    # The generator writes the padded index of base + off as (padded index of base) + constant
+    # when off is a multiple of the padding period, and in full otherwise: both forms must name
+    # the address phys(base + off) = (base + off) + (((base + off) >> ps) << pl).
+    from turbofft_amd.codegen.fft_codegen import KernelEmitter
+    em = KernelEmitter.__new__(KernelEmitter)          # the two methods use no state
+    ps, pl = pad
+    phys = (lambda a: a) if ps < 0 else (lambda a: a + ((a >> ps) << pl))
+    rng = np.random.default_rng(ps * 10 + pl + 100)
+    for off in [0, 1, 7, 32, 96, 256, 1024, 1056, 4096, 31 * 1024, 8 * 4096 + 64]:
+        expr = em.lds_index_at("b0", "b0p", off, pad)
+        for b0 in [0, 1, 31, 32, 33, 1023] + [int(v) for v in rng.integers(0, 1 << 15, 20)]:
+            got = eval(expr.replace("u", ""), {"b0": b0, "b0p": phys(b0)})      # drop the C suffix of unsigned literals
+            assert got == phys(b0 + off), (pad, off, b0, expr)
