@@ -19,6 +19,13 @@ whole batch.  Prints ONE JSON line:
                  "offline" inside it is the same comparison for separate checksum passes
                  before and after the plain plan (the reference's cufft_ft.h baseline),
                  "groups_of_32" the same with the reference's published group size
+                 "full_table" the same with the reference's own complex checksum table in place of
+                 this build's compact (reduced-precision cotangent) form, for the sizes whose
+                 fault-tolerant kernels read the compact form by default
+  sweep        : the whole metric after the timed region: logN 7..24 x {fp32, fp64} at
+                 logBS+logN=28 (main.cu:114-128, compile.sh:12-29), per case launches, median ms
+                 of >= 10 steps, algorithmic GB/s, fraction of the 8 TB/s peak and the overhead
+                 of the fused checksums at groups of 4 tiles (--no_sweep skips it)
   prewarm_s    : untimed executions before the warm-up steps, by time rather than by count:
                  a device that has been idle clocks up over its first tenths of a second
   vendor_baseline : hipFFT (rocFFT) on the same buffers and workload, after the timed
@@ -127,12 +134,28 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
     return res, x, out
 
 
-def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param, thread_bs=4, rounds=7, block=10):
+def make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact=True):
+    """Fault-tolerant plan; compact=False keeps the full (complex) checksum table for every
+    launch (the library reads TURBOFFT_COMPACT_CHECKSUM when a plan is created)."""
+    if compact:
+        return turbofft_amd.TurboFFT(logN, datatype, if_ft=1, thread_bs=thread_bs, param_csv=param)
+    old = os.environ.get("TURBOFFT_COMPACT_CHECKSUM")
+    os.environ["TURBOFFT_COMPACT_CHECKSUM"] = "0"
+    try:
+        return turbofft_amd.TurboFFT(logN, datatype, if_ft=1, thread_bs=thread_bs, param_csv=param)
+    finally:
+        if old is None:
+            del os.environ["TURBOFFT_COMPACT_CHECKSUM"]
+        else:
+            os.environ["TURBOFFT_COMPACT_CHECKSUM"] = old
+
+
+def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param, thread_bs=4, rounds=7, block=10, compact=True):
     """Plain and checksummed plan of the same workload in alternating blocks of `block`
     executions (plain first and last), each block between two events; the overhead is the
     ratio of the median block times, so neither plan is measured on a colder device."""
     plain = turbofft_amd.TurboFFT(logN, datatype, param_csv=param)
-    ft = turbofft_amd.TurboFFT(logN, datatype, if_ft=1, thread_bs=thread_bs, param_csv=param)
+    ft = make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact)
     stream = torch.cuda.current_stream().cuda_stream
     for pl in (plain, ft):
         for _ in range(3):
@@ -152,7 +175,7 @@ def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param,
     for which, e0, e1 in marks:
         times[which].append(e0.elapsed_time(e1) / block)
     counters = {k: v for k, v in ft.ft_counters().items() if k not in ("flagged", "flagged_truncated")}
-    info = {"logNi": ft.logNi, "BS": ft.BS, "n": ft.n, "threads": ft.threads, "lds_bytes": ft.lds_bytes}
+    info = {"logNi": ft.logNi, "BS": ft.BS, "n": ft.n, "threads": ft.threads, "lds_bytes": ft.lds_bytes, "kernels": ft.kernel_names()}
     plain.close()
     ft.close()
     p, f = stats(times[0]), stats(times[1])
@@ -174,6 +197,46 @@ def vendor_case(torch, turbofft_amd, logN, datatype, bs, x, out, reps=20, warmup
     pts = bs * (1 << logN)
     return {"library": "hipFFT", "value": 2 * pts * esize / ms / 1e6, "unit": "GB/s", "ms_per_step": ms,
             "gflops": 5.0 * pts * logN / ms / 1e6, "reps": reps}
+
+
+def sweep_rows(torch, turbofft_amd, lo=7, hi=24, steps=10, ft_rounds=2, ft_block=5, log=None):
+    """The metric's whole range on this device: for each type and logN in [lo, hi] at
+    logBS+logN=28 the plain plan (median of `steps` event-timed steps after a short pre-warm) and
+    the overhead of the fused checksums at groups of 4 tiles (plain and checksummed in
+    alternating blocks).  One input of 2^28 points and one output of 2 x 2^28 per type serve
+    every size."""
+    rows = []
+    stream = torch.cuda.current_stream().cuda_stream
+    for dt in (0, 1):
+        cdt = torch.complex64 if dt == 0 else torch.complex128
+        x = make_input(torch, 1 << (28 - lo), 1 << lo, dt)
+        out = torch.empty(2 << 28, dtype=cdt, device="cuda")
+        for logN in range(lo, hi + 1):
+            bs = 1 << (28 - logN)
+            plan = turbofft_amd.TurboFFT(logN, dt)
+            prewarm(torch, plan, x, out, bs, 0.1)
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+            ev[0].record()
+            for i in range(steps):
+                plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+                ev[i + 1].record()
+            torch.cuda.synchronize()
+            st = stats([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
+            ms = st["median"]
+            row = {"logN": logN, "dtype": "f32" if dt == 0 else "f64", "launches": plan.launches, "ms": ms, "ms_min": st["min"],
+                   "gbs": plan.gbs(bs, ms), "gflops": plan.gflops(bs, ms), "frac": plan.gbs(bs, ms) / HBM_PEAK_GBS,
+                   "frac_per_launch": plan.launches * plan.gbs(bs, ms) / HBM_PEAK_GBS, "steps": steps}
+            plan.close()
+            if ft_rounds > 0:
+                f = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, None, thread_bs=4, rounds=ft_rounds, block=ft_block)
+                row["ft_pct"] = f["overhead_pct"]
+                row["ft_false_alarms"] = f["counters"]["detected"]
+            rows.append(row)
+            if log:
+                log(row)
+        del x, out
+        torch.cuda.empty_cache()
+    return rows
 
 
 def cpu_baseline(logN, datatype, target_s=10.0):
@@ -247,6 +310,8 @@ def main():
     ap.add_argument("--no_ft_overhead", action="store_true",
                     help="skip the extra fault-tolerant run that reports the FT overhead of the workload")
     ap.add_argument("--no_vendor", action="store_true", help="skip the hipFFT side-by-side of the default line")
+    ap.add_argument("--no_sweep", action="store_true", help="skip the logN 7..24 x {fp32, fp64} sweep of the default line")
+    ap.add_argument("--sweep_steps", type=int, default=10, help="timed steps per case of the default line's sweep")
     ap.add_argument("--vendor", action="store_true", help="--sweep: run hipFFT after every case")
     ap.add_argument("--offline", action="store_true", help="--sweep: time the offline checksum scheme after every case")
     ap.add_argument("--membench", action="store_true",
@@ -346,6 +411,16 @@ def main():
         # which this library walks with several blocks per group
         g32 = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param, thread_bs=32, rounds=4)
         ft_line["groups_of_32"] = {"overhead_pct": g32["overhead_pct"], "ms_per_step": g32["ms_per_step"], "order": g32["order"]}
+        # the same groups of 4 with the reference's complex checksum table in every launch (this build's
+        # compact form switched off): what the fused scheme costs on the reference's own arithmetic
+        if any(n.endswith(("_h_ft", "_h2_ft", "_h3_ft")) for n in ft_line["plan"]["kernels"]):
+            full = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param, thread_bs=4, rounds=4, compact=False)
+            ft_line["full_table"] = {"overhead_pct": full["overhead_pct"], "ms_per_step": full["ms_per_step"], "order": full["order"],
+                                     "kernels": full["plan"]["kernels"]}
+        else:
+            ft_line["full_table"] = {"overhead_pct": ft_line["overhead_pct"], "ms_per_step": ft_line["ms_per_step"],
+                                     "note": "this size's fault-tolerant kernels read the full table by default"}
+        ft_line["table"] = "compact" if "kernels" in ft_line["full_table"] else "full"
         # the offline scheme on the same workload: checksum pass, plain plan, checksum pass, compare
         try:
             oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 10),
@@ -363,6 +438,12 @@ def main():
     if not a.no_vendor:
         vendor_line = vendor_case(torch, turbofft_amd, logN, dt, bs, x, out, reps=max(10, a.steps // 10))
     del x, out
+    torch.cuda.empty_cache()
+    sweep = None
+    if not a.no_sweep and not (a.if_ft or a.if_err):
+        t_sw = time.perf_counter()
+        sweep = sweep_rows(torch, turbofft_amd, a.sweep_lo, a.sweep_hi, max(10, a.sweep_steps))
+        sweep_s = time.perf_counter() - t_sw
     tname = "fp32" if dt == 0 else "fp64"
     launches = r["launches"]
     # dominant kernel: with one launch it is the whole step; with several, the launches are
@@ -383,8 +464,12 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((dt, logN, bs, int(bool(a.if_ft or a.if_err)))),
+                     "traffic_source": "constant from the rocprofv3 FETCH_SIZE/WRITE_SIZE runs listed in profiles/, not measured in this run",
                      "kernel_ms": kernel_ms, "alg_bytes_per_launch": r["alg_bytes"]},
     }
+    if sweep is not None:
+        line["sweep"] = sweep
+        line["sweep_s"] = sweep_s
     if sync_ms is not None:
         line["ms_per_step_sync_each_launch"] = sync_ms          # main.cu:53-62 protocol, reported only
     if a.if_ft or a.if_err:

@@ -1222,12 +1222,20 @@ class KernelEmitter:
             c("}")
         else:
             c(f"{{ {R}* q = ps + slot0 + (unsigned long long)part * {4 * T}ull + tx; tfft_ps_store(q, fin1); tfft_ps_store(q + {T}, fin2); tfft_ps_store(q + {2 * T}, fo1); tfft_ps_store(q + {3 * T}, fo2); }}")
-            c("__syncthreads();                       // every wave has waited for its stores: the sums are in memory before the ticket is taken")
+            # Ordering of the hand-off.  The sums are written with agent-scope atomic stores, which go
+            # through the XCD's L2 to memory; a wave's vector-memory counter reaches zero only when every
+            # store it issued has been acknowledged there.  __syncthreads() alone is a workgroup-scope
+            # fence and is not required to wait for outstanding global stores, so each wave waits for its
+            # own (TFFT_WAIT_VMEM) before the barrier; thread 0 takes the ticket after the barrier, i.e.
+            # after every store of the block is in memory.  The deciding block reads the slots with
+            # agent-scope atomic loads (never served from its own L2) issued after its ticket returned.
+            c("TFFT_WAIT_VMEM();")
+            c("__syncthreads();")
             c(f"unsigned* lastp = (unsigned*)(lds_raw + {sp.red_off_bytes});")
             c("if (tx == 0) {")
             c("    const unsigned ticket = atomicAdd(&a.ft.tickets[bx], 1u);")
             c("    lastp[0] = ticket == nparts - 1 ? 1u : 0u;")
-            c("    if (ticket == nparts - 1) a.ft.tickets[bx] = 0u;      // every part has come by: ready for the next launch")
+            c("    if (ticket == nparts - 1) tfft_ps_store(&a.ft.tickets[bx], 0u);      // every part has come by: ready for the next launch (an atomic store like every other access to the word)")
             c("}")
             c("__syncthreads();")
             c("const bool last = lastp[0] != 0u;")

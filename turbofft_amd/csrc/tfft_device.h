@@ -111,6 +111,10 @@ __device__ __forceinline__ float tfft_ckh(unsigned w, int hi) {
 // past the XCD's own L2 to memory.  With them the hand-off needs no device-scope fence -- on this
 // part a release writes the whole L2 back and an acquire invalidates it, and thousands of blocks
 // doing that per launch made the launch four to six times slower.
+// What orders the hand-off instead: every wave waits until its own stores have been acknowledged
+// (TFFT_WAIT_VMEM: vector-memory counter zero, the other counters left alone) before the block
+// barrier that precedes the ticket; an acknowledged agent-scope store is in memory.
+#define TFFT_WAIT_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)     // gfx9 encoding: vmcnt = 0, expcnt = 7, lgkmcnt = 15 (no wait)
 template <typename T> __device__ __forceinline__ void tfft_ps_store(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 template <typename T> __device__ __forceinline__ T tfft_ps_load(const T* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 // a thread's compact-table words parked in LDS behind the exchange buffer, four to an access
@@ -232,9 +236,8 @@ template <int MASK> TFFT_DEV double xl_r(double v) {
 #define XLANE(i, MASK, dst) { dst.x = xl_r<MASK>(r[i].x); dst.y = xl_r<MASK>(r[i].y); }
 #define SNAP()
 
-// Sum over the 64 lanes of a wavefront; every lane receives the total.
-// Steps 1 and 2 are DPP quad permutes, 4/8/16 go through the ds_swizzle
-// crossbar (no LDS memory is touched), 32 uses a permute across the two halves.
+// Sum over the 64 lanes of a wavefront; every lane receives the total: six butterfly steps
+// of __shfl_xor (a ds_bpermute each; no LDS memory is touched).
 TFFT_DEV float wave_sum(float v) {
     v += __shfl_xor(v, 1, 64);
     v += __shfl_xor(v, 2, 64);
