@@ -338,9 +338,15 @@ def main():
         for _ in range(20):
             turbofft_amd.membench(0, src.data_ptr(), dst.data_ptr(), nbytes, 0, 10, st)      # clock the device up
         res = {}
-        for mode, name, moved in ((0, "copy_8B_lanes", 2), (1, "copy_16B_lanes", 2), (2, "read_only", 1), (3, "write_only", 1)):
-            ms = sorted(turbofft_amd.membench(mode, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))
-            res[name] = {"ms_per_pass_median": ms[2], "ms_min": ms[0], "ms_max": ms[4], "GB/s": moved * nbytes / ms[2] / 1e6}
+        # every kernel plain, then with what the FFT kernels use: non-temporal accesses (+4), XCD-aware
+        # tile order (+8) and a bound on the blocks resident per CU (+16*k; the exchange buffer of an
+        # FFT kernel bounds it to 2-4)
+        flavours = (("", 0), ("_nt", 4), ("_nt_xcd", 12), ("_nt_xcd_2percu", 12 + 32), ("_nt_xcd_3percu", 12 + 48), ("_nt_xcd_4percu", 12 + 64), ("_nt_xcd_6percu", 12 + 96))
+        for kind, name, moved in ((0, "copy_8B_lanes", 2), (1, "copy_16B_lanes", 2), (2, "read_only", 1), (3, "write_only", 1)):
+            for sfx, bits in flavours:
+                ms = sorted(turbofft_amd.membench(kind + bits, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))
+                res[name + sfx] = {"ms_per_pass_median": ms[2], "ms_min": ms[0], "ms_max": ms[4], "GB/s": moved * nbytes / ms[2] / 1e6}
+                print(f"{name + sfx:32s} {ms[2]:.4f} ms  {moved * nbytes / ms[2] / 1e6:7.0f} GB/s", file=sys.stderr, flush=True)
         print(json.dumps({"membench": res, "bytes": nbytes, "tile_bytes": 65536, "threads": 256}), flush=True)
         return 0
     if a.sweep:

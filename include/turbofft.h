@@ -128,8 +128,10 @@ int turbofft_time_sync(turbofft_plan_t* plan, const void* in_d, void* out_d, lon
 
 /* Like turbofft_time, with HIP events around every launch of the plan:
  * ms_per_launch[i] receives the mean duration of launch i (entries beyond the
- * plan's launch count are set to 0).  No counterpart in the reference, which
- * times whole plans only (main.cu:52-67). */
+ * plan's launch count are set to 0).  Always times the plan's own row (the one
+ * turbofft_plan_info describes), also for a batch that turbofft_exec would hand
+ * to the small-batch row.  No counterpart in the reference, which times whole
+ * plans only (main.cu:52-67). */
 int turbofft_time_launches(turbofft_plan_t* plan, const void* in_d, void* out_d, long long bs,
                            int warmup, int reps, void* stream, float ms_per_launch[3]);
 
@@ -145,17 +147,25 @@ int turbofft_plan_info(const turbofft_plan_t* plan, int* launches, int logNi[3],
  * (0: none).  Results meet the same accuracy bar; they are not bit-identical to the large-batch
  * row's, whose decomposition differs.  Buffers are unchanged (`out` as documented above).  For
  * the sizes whose large-batch row is a single launch the intermediate of the two launches is a
- * buffer the plan owns: executions of the SAME plan that overlap in time (two streams, two
- * threads) with such a batch race on it -- use one plan per stream, or switch the small-batch
- * row off with turbofft_plan_set_small_batch(plan, 0).  No counterpart in the reference, which
- * has one row per size (main.cu:99,123). */
+ * buffer the plan owns, one per stream: the first is allocated with the plan, a further stream
+ * gets its own at its first small batch (up to 8 per plan; a stream beyond that, or one that is
+ * being captured into a graph and has none yet, runs the large-batch row instead).  Executions
+ * on different streams therefore never share an intermediate; two host threads must not issue
+ * small batches of one plan on the SAME stream at once.  turbofft_plan_set_small_batch(plan, 0)
+ * switches the row off.  No counterpart in the reference, which has one row per size
+ * (main.cu:99,123). */
 long long turbofft_plan_small_batch_max(const turbofft_plan_t* plan);
 int turbofft_plan_set_small_batch(turbofft_plan_t* plan, int enable);
+/* What a batch of `bs` transforms actually runs (the small-batch row up to its cap, else the
+ * plan's own row, which turbofft_plan_info / _grid / _kernel_name describe): its number of
+ * launches and the kernel of each. */
+int turbofft_plan_launches_for_batch(const turbofft_plan_t* plan, long long bs);
+const char* turbofft_plan_kernel_name_for_batch(const turbofft_plan_t* plan, int launch, long long bs);
 
 /* Name of the kernel that launch `launch` of a forward execution runs with the plan's current
  * settings (correction scheme, checksum table, threshold); the role of reading
- * TurboFFT_Kernel_Entry's table entry (TurboFFT.h:22-25).  For batches served by the
- * small-batch row the kernels are that row's. */
+ * TurboFFT_Kernel_Entry's table entry (TurboFFT.h:22-25).  Describes the plan's own row;
+ * turbofft_plan_kernel_name_for_batch tells what a given batch runs. */
 const char* turbofft_plan_kernel_name(const turbofft_plan_t* plan, int launch);
 
 /* Grid size of launch `launch` for `bs` transforms (main.cu:32). */
@@ -177,9 +187,10 @@ int turbofft_plan_set_tb_gap(turbofft_plan_t* plan, int launch, int tb_gap);
  * another block, perhaps on another XCD; the kernel boundary orders the two stores), which
  * returns at once when nothing was located.  Default 8 tiles per block (TURBOFFT_FT_PART_LEN
  * at plan creation overrides; 0 = one block per group, as the reference), so groups of 16 and
- * more are shared; recompute-correcting kernels that do not prefetch only.  The slots are
- * sized at plan creation (128 MiB, plans with thread_bs above the default only) and an
- * execution that would need more runs one block per group.  turbofft_plan_grid keeps returning
+ * more are shared; recompute-correcting kernels that do not prefetch only.  The slots (128 MiB
+ * and 12 MiB of tickets and queue) are allocated by the first execution that shares a group;
+ * an execution that would need more, or whose stream is being captured into a graph before
+ * the slots exist, runs one block per group.  turbofft_plan_grid keeps returning
  * the number of groups.  Executions of one fault-tolerant plan must not overlap in time (they
  * share the slots). */
 int turbofft_plan_set_ft_part_len(turbofft_plan_t* plan, int launch, int tiles);
@@ -310,8 +321,11 @@ int turbofft_offline_ft_time(int logN, int datatype, const void* in_d, void* out
 /* ---- streaming kernels of known traffic (measurement only) ----
  * One pass over `bytes` (a multiple of 65536) in 64 KiB tiles per 256-thread block, all loads
  * of a tile issued before its first store, timed like turbofft_time:
- *   mode 0  copy src -> dst, 8-byte lanes      mode 1  copy, 16-byte lanes
- *   mode 2  read src only                      mode 3  write dst only
+ *   mode bits 0-1: 0  copy src -> dst, 8-byte lanes      1  copy, 16-byte lanes
+ *                  2  read src only                      3  write dst only
+ *   mode bit 2 (+4):  non-temporal accesses, as the FFT kernels mark their tile data
+ *   mode bit 3 (+8):  XCD-aware tile order (runs of 16 consecutive tiles per XCD), as the FFT kernels use
+ *   mode bits 4-7 (+16*k): at most k blocks resident per CU (unused LDS reserved per block; 0: no limit)
  * The yardsticks the FFT kernels are compared with, and kernels of known size for scaling
  * hardware traffic counters.  No counterpart in the reference. */
 int turbofft_membench(int mode, const void* src_d, void* dst_d, size_t bytes, int warmup, int reps,

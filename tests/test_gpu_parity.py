@@ -475,6 +475,69 @@ def test_plans_on_concurrent_streams():
         p.close()
 
 
+def test_small_batches_of_one_plan_on_several_streams():
+    # fp32 2^13 is a single launch for large batches; its small-batch row runs two launches through an
+    # intermediate buffer the plan owns -- one per stream, so executions of ONE plan on different
+    # streams do not share it (ten streams: more than the plan keeps buffers for, the rest run the main row)
+    torch = _torch()
+    dt, logN = "float2", 13
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    cap = plan.small_batch_max()
+    assert cap >= 1 and plan.launches == 1
+    bs = min(cap, 4)
+    small_names, main_names = plan.kernel_names_for_batch(bs), plan.kernel_names_for_batch(cap + 1)
+    assert len(small_names) == 2 and main_names == plan.kernel_names() and small_names != main_names
+    xs = [torch.from_numpy(make(bs, 1 << logN, dt, 200 + i)).cuda() for i in range(10)]
+    want = [torch.from_numpy(O.fft_ref(x.cpu().numpy())) for x in xs]
+    outs = [torch.zeros_like(x) for x in xs]
+    streams = [torch.cuda.Stream() for _ in xs]
+    torch.cuda.synchronize()
+    for rep in range(10):
+        for x, o, st in zip(xs, outs, streams):
+            plan.exec(x.data_ptr(), o.data_ptr(), bs, st.cuda_stream)
+    torch.cuda.synchronize()
+    for o, w in zip(outs, want):
+        assert O.rel_l2(o.cpu().numpy(), w.numpy()) <= O.tolerance(dt, logN)
+    # the same input gives the same bits on every stream that has a buffer of its own (the first eight)
+    o2 = torch.zeros_like(outs[0])
+    plan.exec(xs[0].data_ptr(), o2.data_ptr(), bs, streams[3].cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, outs[0])
+    # (the streams beyond the eighth ran the large-batch row: same transform, held to the same bar above)
+    # per-launch timing describes the plan's own row (one launch), whatever the batch
+    ms = plan.time_launches(xs[0].data_ptr(), outs[0].data_ptr(), bs, 1, 3)
+    assert len(ms) == 1 and ms[0] > 0
+    plan.close()
+
+
+def test_capture_before_the_shared_group_slots_exist():
+    # a fault-tolerant plan with groups of 32 tiles allocates the slots its blocks share a group through at the first
+    # execution that needs them; when that first execution is a graph capture nothing can be allocated, the captured
+    # launches walk whole groups instead, and the replays are still right and still counted
+    torch = _torch()
+    dt, logN, bs = "float2", 12, 300
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=1, thread_bs=32)
+    x = torch.from_numpy(make(bs, 1 << logN, dt, 7)).cuda()
+    out = torch.empty(plan.out_elems(bs), dtype=torch.complex64, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream().cuda_stream)
+    for rep in range(2):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert O.rel_l2(out[: bs << logN].view(bs, -1).cpu().numpy(), O.fft_ref(x.cpu().numpy())) <= O.tolerance(dt, logN)
+    eager = plan.fft(x).clone()            # allocates the slots and shares the groups
+    torch.cuda.synchronize()
+    assert torch.equal(eager, out[: bs << logN].view(bs, -1))
+    c = plan.ft_counters()
+    assert c["detected"] == 0 and c["checked"] == 3 * plan.grid(0, bs)
+    plan.close()
+
+
 def test_cli_vendor_modes():
     # --if_bench 12: the vendor library alone, same line format (cufft.h:45); --if_verify adds the
     # comparison with its result after the one with the host FFT

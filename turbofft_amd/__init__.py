@@ -76,6 +76,9 @@ def lib() -> C.CDLL:
     L.turbofft_plan_set_small_batch.argtypes = [vp, i]
     L.turbofft_plan_kernel_name.argtypes = [vp, i]
     L.turbofft_plan_kernel_name.restype = C.c_char_p
+    L.turbofft_plan_launches_for_batch.argtypes = [vp, ll]
+    L.turbofft_plan_kernel_name_for_batch.argtypes = [vp, i, ll]
+    L.turbofft_plan_kernel_name_for_batch.restype = C.c_char_p
     L.turbofft_plan_tb_gap.argtypes = [vp, i]
     L.turbofft_plan_set_tb_gap.argtypes = [vp, i, i]
     L.turbofft_plan_set_ft_part_len.argtypes = [vp, i, i]
@@ -189,7 +192,8 @@ def offline_ft_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, war
 
 def membench(mode: int, src_ptr: int, dst_ptr: int, nbytes: int, warmup: int = 2, reps: int = 10, stream: int = 0) -> float:
     """ms per pass of a streaming kernel of known traffic: 0 copy with 8-byte lanes, 1 copy with
-    16-byte lanes, 2 read only, 3 write only (measurement yardsticks, not part of any transform)."""
+    16-byte lanes, 2 read only, 3 write only; +4 non-temporal accesses, +8 XCD-aware tile order,
+    +16*k at most k blocks per CU (measurement yardsticks, not part of any transform)."""
     ms = C.c_float(0)
     _check(lib().turbofft_membench(mode, src_ptr, dst_ptr, nbytes, warmup, reps, stream, C.byref(ms)))
     return ms.value
@@ -259,6 +263,12 @@ class TurboFFT:
     def kernel_names(self) -> List[str]:
         """Kernels the launches of a forward execution run with the current settings."""
         return [(lib().turbofft_plan_kernel_name(self._h, i) or b"").decode() for i in range(self.launches)]
+
+    def kernel_names_for_batch(self, bs: int) -> List[str]:
+        """Kernels a batch of `bs` transforms runs: the small-batch row's up to its cap, else the plan's own."""
+        n = lib().turbofft_plan_launches_for_batch(self._h, bs)
+        _check(min(n, 0))
+        return [(lib().turbofft_plan_kernel_name_for_batch(self._h, i, bs) or b"").decode() for i in range(n)]
 
     def tb_gap(self, launch: int) -> int:
         return lib().turbofft_plan_tb_gap(self._h, launch)

@@ -96,6 +96,9 @@ class KernelSpec:
         self.ck16 = bool(k.ck)      # compact checksum table: one cotangent per element (half precision for fp32, single for fp64)
         if self.ck16 and (int(k.ft) != 1 or k.n % 2 or k.pf):
             raise ValueError(f"{k}: the compact checksum table is for recompute-correcting kernels without prefetch")
+        if self.ck16 and k.dtype == "float2" and k.logNi > 16:
+            # the largest entry, cot(pi/3 + pi m/Ni) next to its pole, is about 3 Ni / pi: over 65504 from Ni = 2^17
+            raise ValueError(f"{k}: half-precision cotangents overflow for sub-FFTs of more than 2^16 points")
         self.split = bool(k.split)
         self.pf = bool(k.pf)        # software prefetch of the next tile into a second register set
         # pf > 1: only the first pf elements of a thread are fetched ahead, and only from the start

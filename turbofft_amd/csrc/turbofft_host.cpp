@@ -13,6 +13,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <mutex>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -73,6 +74,7 @@ constexpr size_t kPartSumsBytes = (size_t)128 << 20;
 constexpr long long kPartTickets = 1ll << 20;
 constexpr int kCuLdsBytes = 160 * 1024;     // LDS of one gfx950 compute unit
 constexpr long long kFixGrid = 256;         // blocks of the launch that recomputes queued tiles
+constexpr size_t kMaxSmallWs = 8;           // intermediate buffers (one per stream) a plan keeps for its small-batch row
 // smallest err_threshold the compact checksum tables serve: half-precision entries (fp32 kernels)
 // leave up to 1e-4 of the checksum magnitude as residual on clean data, single-precision ones
 // (fp64 kernels) 1e-8
@@ -253,10 +255,15 @@ struct turbofft_plan {
     // Small batches (plain built-in plans): a second row of narrow tiles in two launches that
     // spreads few transforms over many CUs.  `small` is a plan of its own for that row; it runs
     // for bs <= small_max_bs.  Its intermediate lives in the upper half of the caller's `out`
-    // when this plan is a multi-launch one too, else in `small_ws` (N * small_max_bs elements).
+    // when this plan is a multi-launch one too, else in a buffer of `small_ws` (N * small_max_bs
+    // elements each).
     turbofft_plan* small = nullptr;
     long long small_max_bs = 0;
-    void* small_ws = nullptr;
+    // one intermediate buffer per stream that has run a small batch (single-launch main rows only):
+    // executions on different streams never share one; the first is allocated with the plan
+    struct SmallWs { void* stream; bool assigned; void* buf; };
+    std::vector<SmallWs> small_ws;
+    std::mutex small_mu;
     bool small_enabled = true;
     bool compact_enabled = true;      // TURBOFFT_COMPACT_CHECKSUM=0 keeps the full-table kernels
 };
@@ -319,7 +326,7 @@ const char* turbofft_kernel_name(int i) {
 void turbofft_plan_destroy(turbofft_plan_t* p) {
     if (!p) return;
     if (p->small) turbofft_plan_destroy(p->small);
-    if (p->small_ws) (void)hipFree(p->small_ws);
+    for (auto& w : p->small_ws) if (w.buf) (void)hipFree(w.buf);
     if (p->tw) (void)hipFree(p->tw);
     for (int i = 0; i < 3; ++i) {
         if (p->tw_lo[i]) (void)hipFree(p->tw_lo[i]);
@@ -423,8 +430,11 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             if (rc) { turbofft_plan_destroy(q); return rc; }
             p->small = q;
             p->small_max_bs = sr.tiles();
-            if (p->launches == 1)
-                HIP_TRY(hipMalloc(&p->small_ws, ((size_t)p->small_max_bs << p->logN) * p->esize));
+            if (p->launches == 1) {
+                void* buf = nullptr;
+                HIP_TRY(hipMalloc(&buf, ((size_t)p->small_max_bs << p->logN) * p->esize));
+                p->small_ws.push_back({nullptr, false, buf});
+            }
             break;
         }
     }
@@ -476,6 +486,9 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
             // flavour stays available for the table modes and thresholds the compact form cannot serve
             const tfft_kernel_entry* kc = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 1, r.split(i) ? 1 : 0, 0, 0, r.wv(i), r.nt(i) & 3, 0, r.ck(i));
             if (!kc) return fail(TURBOFFT_ENOPLAN, "no compiled compact-checksum kernel for launch %d of logN=%d", i, p->logN);
+            // the largest cotangent is about 3*Ni/pi: beyond 2^16 points it leaves the half-precision range
+            if (p->datatype == TURBOFFT_FP32 && r.logNi(i) > 16)
+                return fail(TURBOFFT_ENOPLAN, "launch %d of logN=%d: the half-precision compact checksum table serves sub-FFTs of up to 2^16 points", i, p->logN);
             if (int rc = allow_lds(kc, prop)) return rc;
             k = kc;
         }
@@ -574,14 +587,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
             // (a plan row may name its own length per launch, columns 34-36 of the fault-tolerant table; groups of up to
             // kPartLen tiles are never shared, whatever the row says: sharing them measured slower at most sizes)
             for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = (p->row.gp(i) > 0 && !getenv("TURBOFFT_FT_PART_LEN")) ? p->row.gp(i) : part_len;
-            p->part_sums_bytes = kPartSumsBytes;
-            p->tickets_n = kPartTickets;
-            HIP_TRY(hipMalloc(&p->part_sums, p->part_sums_bytes));
-            HIP_TRY(hipMalloc((void**)&p->tickets, sizeof(unsigned) * (size_t)p->tickets_n));
-            HIP_TRY(hipMemset(p->tickets, 0, sizeof(unsigned) * (size_t)p->tickets_n));
-            HIP_TRY(hipMalloc((void**)&p->fix_list, sizeof(long long) * (size_t)p->tickets_n));
-            HIP_TRY(hipMalloc((void**)&p->fix_ctl, 2 * sizeof(unsigned)));
-            HIP_TRY(hipMemset(p->fix_ctl, 0, 2 * sizeof(unsigned)));
+            // (the slots themselves are allocated by the first execution that shares a group)
         }
     }
     return TURBOFFT_OK;
@@ -666,7 +672,6 @@ int turbofft_plan_set_tb_gap(turbofft_plan_t* p, int launch, int tb_gap) {
 int turbofft_plan_set_ft_part_len(turbofft_plan_t* p, int launch, int tiles) {
     if (!p || launch < 0 || launch >= p->launches || tiles < 0) return fail(TURBOFFT_EINVAL, "bad argument");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
-    if (tiles > 0 && !p->part_sums) return fail(TURBOFFT_EINVAL, "the plan holds no slots for shared groups (thread_bs %d)", p->thread_bs);
     p->ft_part_len[launch] = tiles;
     return TURBOFFT_OK;
 }
@@ -886,6 +891,59 @@ const char* turbofft_plan_kernel_name(const turbofft_plan_t* p, int launch) {
     return k ? k->name : nullptr;
 }
 
+// true while `stream` records into a HIP graph: nothing may be allocated or cleared from the host then
+static bool stream_is_capturing(void* stream) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return st != hipStreamCaptureStatusNone;
+}
+
+// Slots, tickets and queue of checksum groups shared by several blocks: allocated by the first
+// execution that needs them (128 MiB + 12 MiB a plan with short groups, or one that only ever runs
+// small batches, never pays for).  Returns false when they are absent and cannot be made now (the
+// stream is being captured, or the allocation failed): the execution then walks whole groups.
+static bool ensure_part_slots(turbofft_plan* p, void* stream) {
+    if (p->part_sums) return true;
+    if (stream_is_capturing(stream)) return false;
+    void *ps = nullptr, *tk = nullptr, *fl = nullptr, *fc = nullptr;
+    const size_t tn = (size_t)kPartTickets;
+    bool ok = hipMalloc(&ps, kPartSumsBytes) == hipSuccess && hipMalloc(&tk, sizeof(unsigned) * tn) == hipSuccess &&
+              hipMalloc(&fl, sizeof(long long) * tn) == hipSuccess && hipMalloc(&fc, 2 * sizeof(unsigned)) == hipSuccess;
+    // cleared on the stream the execution is issued on, ahead of its kernels
+    ok = ok && hipMemsetAsync(tk, 0, sizeof(unsigned) * tn, (hipStream_t)stream) == hipSuccess &&
+         hipMemsetAsync(fc, 0, 2 * sizeof(unsigned), (hipStream_t)stream) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        if (ps) (void)hipFree(ps);
+        if (tk) (void)hipFree(tk);
+        if (fl) (void)hipFree(fl);
+        if (fc) (void)hipFree(fc);
+        return false;
+    }
+    p->part_sums = ps; p->tickets = (unsigned*)tk; p->fix_list = (long long*)fl; p->fix_ctl = (unsigned*)fc;
+    p->part_sums_bytes = kPartSumsBytes;
+    p->tickets_n = kPartTickets;
+    return true;
+}
+
+// The row a batch of `bs` transforms runs: the small-batch row (plain built-in plans, bs up to its cap) or the plan's own
+static const turbofft_plan* row_for_batch(const turbofft_plan* p, long long bs) {
+    return (p->small && p->small_enabled && bs >= 1 && bs <= p->small_max_bs) ? p->small : p;
+}
+
+int turbofft_plan_launches_for_batch(const turbofft_plan_t* p, long long bs) {
+    if (!p || bs < 0) return fail(TURBOFFT_EINVAL, "bad argument");
+    return row_for_batch(p, bs)->launches;
+}
+
+const char* turbofft_plan_kernel_name_for_batch(const turbofft_plan_t* p, int launch, long long bs) {
+    if (!p || bs < 0) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
+    const turbofft_plan* q = row_for_batch(p, bs);
+    if (launch < 0 || launch >= q->launches) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
+    const tfft_kernel_entry* k = launch_kernel(q, launch, false);
+    return k ? k->name : nullptr;
+}
+
 static bool ranges_overlap(const void* a, size_t an, const void* b, size_t bn) {
     const char *a0 = (const char*)a, *b0 = (const char*)b;
     return a0 < b0 + bn && b0 < a0 + an;
@@ -911,11 +969,32 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         // few transforms: the narrow-tile row, with the caller's workspace half when there is
         // one, else the plan's own intermediate buffer
         exec_opts so = o;
-        if (!so.workspace && p->launches == 1) so.workspace = p->small_ws;
+        bool have_ws = true;
+        if (!so.workspace && p->launches == 1) {
+            // the intermediate of the two narrow-tile launches: a buffer of the plan's, one per stream, so that
+            // executions of one plan on several streams do not share it.  A stream without one gets one now,
+            // unless it is being captured or the plan already keeps kMaxSmallWs: then the main row runs.
+            std::lock_guard<std::mutex> lk(p->small_mu);
+            turbofft_plan::SmallWs* w = nullptr;
+            for (auto& e : p->small_ws) if (e.assigned && e.stream == stream) { w = &e; break; }
+            if (!w) for (auto& e : p->small_ws) if (!e.assigned) { e.assigned = true; e.stream = stream; w = &e; break; }
+            if (!w && p->small_ws.size() < kMaxSmallWs && !stream_is_capturing(stream)) {
+                void* buf = nullptr;
+                if (hipMalloc(&buf, ((size_t)p->small_max_bs << p->logN) * p->esize) == hipSuccess) {
+                    p->small_ws.push_back({stream, true, buf});
+                    w = &p->small_ws.back();
+                } else {
+                    (void)hipGetLastError();
+                }
+            }
+            if (w) so.workspace = w->buf; else have_ws = false;
+        }
+        if (have_ws) {
         if (ranges_overlap(in_d, data_bytes, out, data_bytes * ((p->launches > 1 && !o.workspace) ? 2 : 1)))
             return fail(TURBOFFT_EINVAL, "in [%p, +%zu) overlaps out [%p, ...): the transform is out of place", in_d, data_bytes, (void*)out);
         p->last_stream.store(stream, std::memory_order_release);
         return exec_impl(p->small, in_d, out_d, bs, stream, so);
+        }
     }
     const Row& r = p->row;
     char* work = o.workspace ? (char*)o.workspace : out + data_bytes;
@@ -989,7 +1068,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             // groups longer than ft_part_len tiles: several blocks per group, where the plan's slots suffice
             const long long parts = (a.thread_bs + p->ft_part_len[i] - 1) / p->ft_part_len[i];
             const unsigned long long need = (unsigned long long)grid * parts * 4ull * k->threads * (p->esize / 2);
-            if (need <= p->part_sums_bytes && grid <= p->tickets_n && grid * parts <= 0x7fffffffll) {
+            if (need <= kPartSumsBytes && grid <= kPartTickets && grid * parts <= 0x7fffffffll && ensure_part_slots(p, stream)) {
                 a.ft.parts = (int)parts;
                 a.ft.part_len = p->ft_part_len[i];
                 a.ft.part_sums = p->part_sums;
@@ -1044,7 +1123,9 @@ int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, lo
     if (!p || !ms_per_launch || reps < 1 || warmup < 0 || bs < 1) return fail(TURBOFFT_EINVAL, "bad argument");
     for (int i = 0; i < 3; ++i) ms_per_launch[i] = 0.f;
     for (int i = 0; i < warmup; ++i) {
-        int rc = turbofft_exec(p, in_d, out_d, bs, stream);
+        exec_opts wo;
+        wo.main_row = true;
+        int rc = exec_impl(p, in_d, out_d, bs, stream, wo);
         if (rc) return rc;
     }
     EventSet es;
@@ -1052,6 +1133,7 @@ int turbofft_time_launches(turbofft_plan_t* p, const void* in_d, void* out_d, lo
     if (rc) return rc;
     exec_opts o;
     o.ev = es.ev.data();
+    o.main_row = true;          // the plan's own row whatever the batch: its launches are what the caller gets times for
     for (int r = 0; r < reps; ++r) {
         rc = exec_impl(p, in_d, out_d, bs, stream, o);
         if (rc) return rc;
