@@ -18,7 +18,8 @@ whole batch.  Prints ONE JSON line:
                  the ratio of the two medians (--no_ft_overhead skips it);
                  "offline" inside it is the same comparison for separate checksum passes
                  before and after the plain plan (the reference's cufft_ft.h baseline),
-                 "groups_of_32" the same with the reference's published group size
+                 "groups_of_32" the same with the reference's published group size,
+                 "thread_level" the same for thread-level verification (if_ft = 2)
                  "full_table" the same with the reference's own complex checksum table in place of
                  this build's compact (reduced-precision cotangent) form, for the sizes whose
                  fault-tolerant kernels read the compact form by default
@@ -134,11 +135,12 @@ def run_case(torch, turbofft_amd, logN, datatype, bs, steps, warmup, if_ft=0, if
     return res, x, out
 
 
-def make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact=True):
+def make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact=True, scheme=1):
     """Fault-tolerant plan; compact=False keeps the full (complex) checksum table for every
-    launch (the library reads TURBOFFT_COMPACT_CHECKSUM when a plan is created)."""
+    launch (the library reads TURBOFFT_COMPACT_CHECKSUM when a plan is created); scheme 2 is
+    thread-level verification."""
     if compact:
-        return turbofft_amd.TurboFFT(logN, datatype, if_ft=1, thread_bs=thread_bs, param_csv=param)
+        return turbofft_amd.TurboFFT(logN, datatype, if_ft=scheme, thread_bs=thread_bs, param_csv=param)
     old = os.environ.get("TURBOFFT_COMPACT_CHECKSUM")
     os.environ["TURBOFFT_COMPACT_CHECKSUM"] = "0"
     try:
@@ -150,12 +152,12 @@ def make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact=True):
             os.environ["TURBOFFT_COMPACT_CHECKSUM"] = old
 
 
-def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param, thread_bs=4, rounds=7, block=10, compact=True):
+def interleaved_overhead(torch, turbofft_amd, logN, datatype, bs, x, out, param, thread_bs=4, rounds=7, block=10, compact=True, scheme=1):
     """Plain and checksummed plan of the same workload in alternating blocks of `block`
     executions (plain first and last), each block between two events; the overhead is the
     ratio of the median block times, so neither plan is measured on a colder device."""
     plain = turbofft_amd.TurboFFT(logN, datatype, param_csv=param)
-    ft = make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact)
+    ft = make_ft_plan(turbofft_amd, logN, datatype, thread_bs, param, compact, scheme)
     stream = torch.cuda.current_stream().cuda_stream
     for pl in (plain, ft):
         for _ in range(3):
@@ -231,6 +233,10 @@ def sweep_rows(torch, turbofft_amd, lo=7, hi=24, steps=10, ft_rounds=2, ft_block
                 f = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, None, thread_bs=4, rounds=ft_rounds, block=ft_block)
                 row["ft_pct"] = f["overhead_pct"]
                 row["ft_false_alarms"] = f["counters"]["detected"]
+                # thread-level verification (every tile checked on its own, by its threads)
+                f = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, None, thread_bs=1, rounds=ft_rounds, block=ft_block, scheme=2)
+                row["ft_thread_level_pct"] = f["overhead_pct"]
+                row["ft_false_alarms"] += f["counters"]["detected"]
             rows.append(row)
             if log:
                 log(row)
@@ -427,6 +433,11 @@ def main():
             ft_line["full_table"] = {"overhead_pct": ft_line["overhead_pct"], "ms_per_step": ft_line["ms_per_step"],
                                      "note": "this size's fault-tolerant kernels read the full table by default"}
         ft_line["table"] = "compact" if "kernels" in ft_line["full_table"] else "full"
+        # thread-level verification of the same workload: every thread checks its own register-level DFTs,
+        # every tile is decided before it is stored (no groups)
+        tl = interleaved_overhead(torch, turbofft_amd, logN, dt, bs, x, out, a.param, thread_bs=1, rounds=4, scheme=2)
+        ft_line["thread_level"] = {"overhead_pct": tl["overhead_pct"], "ms_per_step": tl["ms_per_step"], "order": tl["order"],
+                                   "kernels": tl["plan"]["kernels"], "counters": tl["counters"]}
         # the offline scheme on the same workload: checksum pass, plain plan, checksum pass, compare
         try:
             oms, oflag = turbofft_amd.offline_ft_time(logN, dt, x.data_ptr(), out.data_ptr(), bs, 2, max(10, a.steps // 10),

@@ -49,7 +49,21 @@ const char* turbofft_last_error(void);
  * twiddle table of initializeData (initializeData.h:31-37) and the DFT
  * checksum table (abft.h:21-61, main.cu:85-93).
  *   datatype   TURBOFFT_FP32 / TURBOFFT_FP64
- *   if_ft      1: fault-tolerant kernels (fused two-sided checksums)
+ *   if_ft      1: fault-tolerant kernels (fused two-sided checksums over groups of
+ *              thread_bs tiles: the scheme of the reference's current generator,
+ *              fft_codegen.py:354-384,432-503)
+ *              2: thread-level verification (the scheme of the reference's
+ *              data_ft/ft_scheme_thread_bs=1_* tables, of which its generator keeps only the
+ *              per-thread sums; the command line's --ft_scheme 1): every thread applies the same
+ *              two-sided checksum (output side r[o%3], input side c_R = W_R^T r, abft.h:21-61)
+ *              to the radix-R DFTs it computes in registers, pass by pass, and objects when
+ *              |in - out| / (err_smoothing + |in| + |out|) > err_threshold for its two sums;
+ *              nothing is summed across threads, the block only agrees on whether any thread
+ *              objected, and a tile one did object to is recomputed before it is stored
+ *              (bit-identical to an undisturbed run; correct = 0 stores it as computed).
+ *              Every tile is its own group: `checked` counts tiles, the flagged list names
+ *              them, thread_bs only shapes the grid and the injection cadence.  Runs the plain
+ *              plan rows; no checksum table, no delayed correction.
  *   if_err     1: inject errors with the reference cadence and correct them
  *              (implies if_ft, CommandLineParser.h:66-68)
  *   thread_bs  tiles per block = checksum group size (--thread_bs).  Without

@@ -36,6 +36,14 @@ Parity status (what pins each function):
                           injected error and the "clean data -> no detection"
                           invariant.  The reference holds no vectors for it.
 
+  thread_level_model      the same two-sided checksum applied by each thread to its own
+                          register-level DFTs (the reference keeps the per-thread sums and the
+                          result tables of its thread-level scheme, not its code); pinned by the
+                          checksum identity against brute-force DFTs, by the closed-form shift of
+                          an injected error (one thread of one pass objects, by exactly
+                          injected_delta_closed_form of the first radix) and by faults put on
+                          single butterfly outputs of every pass.
+
 The reference repository ships no golden vectors, known-answer tests or
 fixtures for this path (its only check is a run-time comparison with cuFFT),
 so every pin above is mathematical.
@@ -694,6 +702,119 @@ def ft_plan_model(x: np.ndarray, row: PlanRow, dtype, thread_bs: int, tb_gap: Se
         decisions.append(ft_launch_model(xin, yout, geom.n, groups, dtype, c_vec,
                                          err_smoothing, err_threshold))
     return decisions, out
+
+
+# --------------------------------------------------------------------------
+# thread-level verification
+# --------------------------------------------------------------------------
+def thread_level_vectors(R: int, dtype) -> Tuple[np.ndarray, np.ndarray]:
+    """Checksum vectors of one register-level radix-R DFT: the output-side r[o % 3]
+    (abft.h:22-28) and the input-side c_R = W_R^T r (abft.h:45-60 for N = R, exact angles)."""
+    ct = _ctype(dtype)
+    rv = checksum_r(np.complex128)[np.arange(R) % 3]
+    return np.fft.fft(rv).astype(ct), rv.astype(ct)
+
+
+@dataclass
+class ThreadVerdict:
+    tile: int
+    s: int          # sub-FFT of the tile
+    q: int          # pass
+    thread: int     # thread of the sub-FFT (x = 0 .. Ni/n - 1)
+    delta: float    # in - out of the thread's two sums
+    mag: float      # |in| + |out|
+    ratio: float    # |delta| / (err_smoothing + mag)
+
+
+def thread_level_model(xin: np.ndarray, n: int, dtype, injections: Optional[Sequence[Injection]] = None,
+                       out_faults: Optional[Sequence[Tuple[int, int, int, int, int, complex]]] = None,
+                       err_smoothing: float = ERR_SMOOTHING_DEFAULT, err_threshold: float = ERR_THRESHOLD_DEFAULT):
+    """Thread-level verification of one launch (the scheme behind the reference's
+    data_ft/ft_scheme_thread_bs=1_* tables, of which its generator keeps only the per-thread
+    sums, fft_codegen.py:354-384): the two-sided checksum of abft.h applied by every thread to
+    the radix-R DFTs it computes in registers, pass by pass.
+
+    xin[tile, s, m]: launch inputs.  In pass q a thread x of sub-FFT s owns the U = n/R DFTs
+    `rest = x + (Ni/n) u` (rest = low + P j: inputs m = j + J i of the length-M sub-problem `low`).
+      in  = sum over its DFTs and their inputs  of re+im(x_i c_R[i])
+      out = sum over its DFTs and their outputs of re+im(y_o r[o % 3])   (before the pass's twiddles)
+      the thread objects iff |in - out| / (err_smoothing + |in| + |out|) > err_threshold
+    A tile is flagged when any of its threads objects in any pass; it is then recomputed, so the
+    corrected result is the clean transform.  `injections` add `mag` to re of input element m
+    (m < Ni/n: register 0 of thread m) of sub-FFT s after the first pass's input sums
+    (fft_codegen.py:412-415); `out_faults` (tile, s, q, rest, o, value) add `value` to output o of one
+    register-level DFT of pass q before the output sums (a fault inside that butterfly network).
+    Returns (flagged[tile] bool array, list of ThreadVerdict for the objecting threads, worst ratio
+    among the threads that did not object)."""
+    ct = _ctype(dtype)
+    rt = _rtype(dtype)
+    xin = np.asarray(xin).astype(ct)
+    ntile, BS, Ni = xin.shape
+    Tr = Ni // n
+    tw = twiddle_table(Ni, dtype)
+    P, M = 1, Ni
+    data = xin.reshape(ntile, BS, M, P)
+    passes = radix_passes(Ni, n)
+    flagged = np.zeros(ntile, dtype=bool)
+    verdicts: List[ThreadVerdict] = []
+    worst_quiet = 0.0
+    for q, R in enumerate(passes):
+        J = M // R
+        U = n // R
+        cR, rR = thread_level_vectors(R, dtype)
+        d = np.moveaxis(data.reshape(ntile, BS, R, J, P), 2, 0).copy()        # [i, tile, s, j, low]
+        t = (d * cR.reshape(R, 1, 1, 1, 1)).astype(ct)
+        sin = (t.real + t.imag).astype(rt).sum(axis=0, dtype=rt)                # [tile, s, j, low]
+        if q == 0 and injections:
+            for inj in injections:
+                assert 0 <= inj.m < Tr, "the injected element is one of the first Ni/n of its sub-FFT"
+                d[0, inj.tile, inj.s, inj.m, 0] += rt.type(inj.mag)
+        y = _reg_fft(d, R, ct)                                                  # [o, tile, s, j, low]
+        if out_faults:
+            for (ft_tile, ft_s, ft_q, ft_rest, ft_o, ft_val) in out_faults:
+                if ft_q == q:
+                    y[ft_o, ft_tile, ft_s, ft_rest // P, ft_rest % P] += ct.type(ft_val)
+        t = (y * rR.reshape(R, 1, 1, 1, 1)).astype(ct)
+        sout = (t.real + t.imag).astype(rt).sum(axis=0, dtype=rt)
+        # DFT (j, low) is `rest = low + P j` = x + Tr u of thread x
+        tin = sin.reshape(ntile, BS, U, Tr).sum(axis=2, dtype=rt)
+        tout = sout.reshape(ntile, BS, U, Tr).sum(axis=2, dtype=rt)
+        delta = (tin - tout).astype(np.float64)
+        mag = (np.abs(tin) + np.abs(tout)).astype(np.float64)
+        ratio = np.abs(delta) / (err_smoothing + mag)
+        bad = ratio > err_threshold
+        for (ti, si, xi) in zip(*np.nonzero(bad)):
+            verdicts.append(ThreadVerdict(int(ti), int(si), q, int(xi), float(delta[ti, si, xi]), float(mag[ti, si, xi]),
+                                          float(ratio[ti, si, xi])))
+        flagged |= bad.any(axis=(1, 2))
+        if (~bad).any():
+            worst_quiet = max(worst_quiet, float(ratio[~bad].max()))
+        if q != len(passes) - 1:
+            delta_w = tw[M - 1 + np.arange(J)].astype(ct)
+            angle = np.ones(J, dtype=ct)
+            for o in range(1, R):
+                angle = _zmul(angle, delta_w, ct)
+                y[o] = (y[o] * angle.reshape(1, 1, J, 1)).astype(ct)
+        data = np.moveaxis(y, 0, 3).reshape(ntile, BS, J, R * P)               # [tile, s, j, o, low] -> low' = low + P o
+        P *= R
+        M = J
+    return flagged, verdicts, worst_quiet
+
+
+def thread_level_plan_model(x: np.ndarray, row: PlanRow, dtype, injections: Optional[Sequence[Injection]] = None,
+                            inj_launch: int = -1, err_smoothing: float = ERR_SMOOTHING_DEFAULT,
+                            err_threshold: float = ERR_THRESHOLD_DEFAULT):
+    """thread_level_model for every launch of a plan on clean data plus injected errors (in launch
+    `inj_launch`).  Returns (per launch: flagged[tile], verdicts, worst quiet ratio) and the corrected
+    output (every flagged tile is recomputed, so it is the clean transform)."""
+    out, stages = plan_fft(x, row, dtype, return_stages=True)
+    geoms = launch_geometry(row, x.shape[0])
+    inj_launch = inj_launch % row.launches
+    res = []
+    for li, (geom, (lin, _)) in enumerate(zip(geoms, stages)):
+        res.append(thread_level_model(geom.gather(lin), geom.n, dtype, injections if li == inj_launch else None,
+                                      None, err_smoothing, err_threshold))
+    return res, out
 
 
 # --------------------------------------------------------------------------

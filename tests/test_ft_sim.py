@@ -324,3 +324,109 @@ def test_groups_shared_by_several_blocks(dtype, logNi, BS, n, split, pf, ck, tbs
         assert np.array_equal(many[2], one[2])         # recomputed tiles are bit-identical
         if inj_mode == 1:
             assert one[3][1] > 0                        # the cadence raises detections (long groups may miss some)
+
+
+# ---- thread-level verification (`_tt` kernels) ----
+
+def run_tl(dtype, logNi, BS, n, ntiles, thread_bs, tb_gap, inj_mode, correct, inj_every=1, inj_tile=0, inj_s=0, inj_m=0,
+           mag=100.0, seed=0, split=0, threshold=1e-3, smoothing=1000.0):
+    sp = KernelSpec(KernelKey(dtype, "row1", logNi, BS, n, 3, split))
+    N = 1 << logNi
+    bs = ntiles * BS
+    x = rnd((bs, N), seed).astype(simlib.ctype_of(dtype))
+    ka = simlib.KArgs()
+    ka.ntiles, ka.nrows, ka.thread_bs, ka.tb_gap = ntiles, bs, thread_bs, tb_gap
+    st = simlib.FtState(ka)
+    ka.ft.launch, ka.ft.correct = 0, correct
+    ka.ft.inj_mode, ka.ft.inj_every, ka.ft.inj_tile, ka.ft.inj_s, ka.ft.inj_m, ka.ft.inj_mag = \
+        inj_mode, inj_every, inj_tile, inj_s, inj_m, mag
+    ka.ft.err_smoothing, ka.ft.err_threshold = smoothing, threshold
+    grid = (ntiles + thread_bs - 1) // thread_bs
+    y = simlib.run_sim(sp, x, bs * N, ka, grid, simlib.twiddle_table(N, dtype)).reshape(bs, N)
+    return sp, x, y, st
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("logNi,BS,n,split", [(8, 4, 16, 0), (7, 8, 8, 0), (10, 1, 8, 1), (5, 16, 8, 0), (3, 64, 8, 0), (13, 1, 32, 1)])
+def test_thread_level_verification(dtype, logNi, BS, n, split):
+    """Every thread checks the register-level DFTs of each pass against the checksum vectors of
+    their radix; a tile that a thread objects to is recomputed before it is stored.  Clean data
+    raises nothing; the reference cadence (100 on register 0 of thread 0 of one tile per block,
+    after the input sums) is caught in exactly the injected tiles, as the oracle's model of the
+    scheme says, and the stored result is bit-identical to an undisturbed run."""
+    ntiles, tbs, gap = (24, 4, 3) if logNi < 13 else (6, 2, 2)
+    sp, x, y0, st = run_tl(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=0, correct=1, split=split)
+    assert st.checked == ntiles and st.detected == 0 and not st.pairs()
+    assert O.rel_l2(y0, O.fft_ref(x)) < O.tolerance(dtype, logNi)
+    sp, x, y, st = run_tl(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=1, correct=1, split=split)
+    groups = O.tile_groups(ntiles, tbs, gap)
+    injs = O.reference_injections(groups, tbs, 100.0)
+    flagged, verdicts, quiet = O.thread_level_model(x.reshape(ntiles, BS, -1), n, dtype, injs)
+    assert sorted(np.nonzero(flagged)[0]) == sorted(i.tile for i in injs)          # the model catches every injection
+    assert quiet < 0.1 * 1e-3 and all(v.ratio > 10 * 1e-3 for v in verdicts)       # and nothing sits near the rule
+    assert st.detected == len(injs) and sorted(t for _, t in st.pairs()) == sorted(i.tile for i in injs)
+    assert np.array_equal(y, y0)
+    # detect only: the flagged tile is stored as computed, every output of the hit sub-FFT off by the magnitude
+    sp, x, y, st = run_tl(dtype, logNi, BS, n, ntiles, tbs, gap, inj_mode=1, correct=0, split=split)
+    assert st.detected == len(injs)
+    err = np.abs(y - y0).reshape(ntiles, BS, -1)
+    for inj in injs:
+        assert np.allclose(err[inj.tile, 0], 100.0, rtol=1e-3)
+    assert err[[t for t in range(ntiles) if t not in {i.tile for i in injs}]].max() == 0
+
+
+def test_thread_level_host_chosen_element_and_threshold():
+    # mode 2: one tile, sub-FFT 2, element 11 (register 0 of thread 11); the objecting thread is the model's
+    ntiles, tbs, gap = 20, 5, 2
+    sp, x, y, st = run_tl("float2", 8, 4, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000, inj_tile=13,
+                          inj_s=2, inj_m=11, mag=100.0)
+    assert st.detected == 1 and st.pairs() == [(0, 13)]
+    flagged, verdicts, quiet = O.thread_level_model(x.reshape(ntiles, 4, -1), 16, "float2", [O.Injection(13, 2, 11, 100.0)])
+    assert [(v.tile, v.s, v.q, v.thread) for v in verdicts] == [(13, 2, 0, 11)]
+    assert O.rel_l2(y, O.fft_ref(x)) < O.tolerance("float2", 8)
+    # an error far below the rule stays (model and kernel agree that nobody objects)
+    sp, x, y, st = run_tl("float2", 8, 4, 16, ntiles, tbs, gap, inj_mode=2, correct=1, inj_every=1000, inj_tile=13,
+                          inj_s=2, inj_m=11, mag=0.05)
+    flagged, verdicts, quiet = O.thread_level_model(x.reshape(ntiles, 4, -1), 16, "float2", [O.Injection(13, 2, 11, 0.05)])
+    assert not flagged.any() and quiet < 0.5e-3 and st.detected == 0
+
+
+@pytest.mark.parametrize("dtype,logNi,BS,n,log_ncols", [("double2", 7, 16, 8, 8), ("float2", 8, 16, 16, 6)])
+def test_thread_level_column_kernel(dtype, logNi, BS, n, log_ncols):
+    sp = KernelSpec(KernelKey(dtype, "col", logNi, BS, n, 3))
+    Ni, ncols, outer = 1 << logNi, 1 << log_ncols, 3
+    x = rnd((outer, Ni, ncols), 5)
+    ref = np.fft.fft(x.astype(simlib.ctype_of(dtype)).astype(np.complex128), axis=1)
+    k = np.arange(Ni)[:, None]
+    col = np.arange(ncols)[None, :]
+    ref = ref * np.exp(-2j * np.pi * ((k * col) % (Ni * ncols)) / (Ni * ncols))
+    lo_bits, hi, lo = simlib.split_tables(logNi + log_ncols, dtype)
+    for inj_tile, want in ((7, [(0, 7)]), (1 << 40, [])):
+        ka = simlib.KArgs()
+        ka.ntiles = outer * ncols // BS
+        ka.thread_bs, ka.tb_gap, ka.log_ncols = 3, 2, log_ncols
+        ka.tw_lo_bits = lo_bits
+        st = _ft_args(ka, ka.ntiles, 1, inj_tile, 100.0)
+        y = simlib.run_sim(sp, x, x.size, ka, (ka.ntiles + 2) // 3, simlib.twiddle_table(Ni, dtype), hi, lo).reshape(outer, Ni, ncols)
+        assert st.checked == ka.ntiles and st.pairs() == want and st.detected == len(want)
+        assert O.rel_l2(y, ref) < O.tolerance(dtype, logNi)
+
+
+@pytest.mark.parametrize("dtype,logA,BS,n,logQ,logC", [("double2", 8, 8, 8, 0, 4), ("float2", 8, 16, 16, 3, 4)])
+def test_thread_level_transposing_kernel(dtype, logA, BS, n, logQ, logC):
+    sp = KernelSpec(KernelKey(dtype, "rowT", logA, BS, n, 3))
+    A, Q, Cc = 1 << logA, 1 << logQ, 1 << logC
+    bs = 2
+    x = rnd((bs, Cc, Q, A), 7)
+    xc = x.astype(simlib.ctype_of(dtype)).astype(np.complex128)
+    ref = np.transpose(np.fft.fft(xc, axis=3), (0, 3, 2, 1))
+    ntiles = bs * Q * Cc // BS
+    for inj_tile, want in ((ntiles - 1, [(0, ntiles - 1)]), (1 << 40, [])):
+        ka = simlib.KArgs()
+        ka.ntiles = ntiles
+        ka.thread_bs, ka.tb_gap = 2, 3
+        ka.logQ, ka.logC, ka.logN = logQ, logC, logA + logQ + logC
+        st = _ft_args(ka, ka.ntiles, 1, inj_tile, 100.0)
+        y = simlib.run_sim(sp, x, x.size, ka, (ntiles + 1) // 2, simlib.twiddle_table(A, dtype)).reshape(bs, A, Q, Cc)
+        assert st.checked == ntiles and st.pairs() == want and st.detected == len(want)
+        assert O.rel_l2(y, ref) < O.tolerance(dtype, logA)

@@ -633,3 +633,76 @@ def test_groups_shared_by_several_blocks(dt, logN, bs, tbs):
         assert np.array_equal(ys, y) and np.array_equal(ys0, y0) and np.array_equal(ys, ys0)
     assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
     plan.close()
+
+
+# ---- thread-level verification (if_ft = 2) ----
+
+TL_CASES = [("float2", 10, 64), ("double2", 10, 16), ("float2", 13, 32), ("double2", 15, 8), ("float2", 16, 4),
+            ("float2", 21, 1), ("double2", 20, 2), ("float2", 24, 1), ("float2", 5, 1000), ("double2", 3, 777),
+            ("float2", 15, 6), ("double2", 14, 5)]
+
+
+@pytest.mark.parametrize("dt,logN,bs", TL_CASES)
+@pytest.mark.parametrize("tbs", [1, 4])
+def test_thread_level_verification_matches_oracle_model(dt, logN, bs, tbs):
+    # if_ft = 2: every thread checks the register-level DFTs of each pass on its own; no sums cross
+    # threads, a tile a thread objects to is recomputed before it is stored.  Clean data raises
+    # nothing; the reference's own injection (100 on element 0 of one tile per block of the last
+    # launch, after the input sums) is caught in exactly the tiles the oracle's model of the scheme
+    # flags, and the stored result is bit-identical to an undisturbed run.  A thread's two sums grow
+    # with the data of its launch, not with the tile or the group, so 100 stays visible far beyond the
+    # 2^10 points where the block-level sums hide it; only where the model puts it near the rule (the
+    # last launch of the three-launch plans, whose inputs have grown to a few hundred) the test takes
+    # a larger magnitude.
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=2, if_err=1, thread_bs=tbs)
+    assert all(n.endswith("_tt") for n in plan.kernel_names()), plan.kernel_names()
+    gaps = [7, 5, 3][:plan.launches]
+    for i, g in enumerate(gaps):
+        plan.set_tb_gap(i, g)
+    x = make(bs, 1 << logN, dt, logN + 21)
+    row = O.PlanRow.from_list(plan.plan_row())
+    geoms = O.launch_geometry(row, bs)
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    assert c0["detected"] == 0 and c0["flagged"] == [] and c0["checked"] == sum(g.ntiles for g in geoms)
+    assert O.rel_l2(y0, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    last = plan.launches - 1
+    groups = O.tile_groups(geoms[last].ntiles, tbs, gaps[last])
+    for mag in (100.0, 1.0e4, 1.0e6):
+        injs = O.reference_injections(groups, tbs, mag)
+        res, _ = O.thread_level_plan_model(x, row, dt, injs)
+        model = sorted((li, int(t)) for li, (fl, _, _) in enumerate(res) for t in np.nonzero(fl)[0])
+        # nothing near the rule: every injection well above it, every other thread well below
+        if model == sorted((last, i.tile) for i in injs) and all(quiet < 0.1e-3 and all(v.ratio > 5e-3 for v in verdicts) for _, verdicts, quiet in res):
+            break
+    else:
+        pytest.fail("no magnitude keeps this case away from the rule")
+    print(f"thread-level case: magnitude {mag:g}, {len(injs)} injections", flush=True)
+    assert mag == 100.0 or plan.launches == 3
+    plan.set_injection(1, mag=mag)
+    y, c = run(plan, x)
+    want = model if len(model) <= 4096 else None
+    assert c["detected"] == len(injs) == c["corrected"] and c["uncorrectable"] == 0
+    if want is not None and not c["flagged_truncated"]:
+        assert sorted(c["flagged"]) == want
+    assert np.array_equal(y, y0)
+    # detect only: the tiles are stored as computed
+    plan.set_ft_params(1000.0, 1e-3, correct=0)
+    y1, c1 = run(plan, x)
+    assert c1["detected"] == len(injs) and c1["corrected"] == 0 and not np.array_equal(y1, y0)
+    plan.close()
+
+
+def test_thread_level_verification_in_an_earlier_launch_and_refusals():
+    plan = turbofft_amd.TurboFFT(16, "float2", if_ft=2, thread_bs=2)
+    plan.set_ft_params(1000.0, 1e-3, correct=1)
+    plan.set_injection(2, launch=0, every=1 << 30, tile_phase=9, s=3, m=1, mag=100.0)
+    x = make(6, 1 << 16, "float2", 5)
+    y, c = run(plan, x)
+    assert c["flagged"] == [(0, 9)] and c["corrected"] == 1
+    assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance("float2", 16)
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        plan.set_ft_params(1000.0, 1e-3, correct=2)          # no delayed correction: the tile never left the registers
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        plan.set_checksum_mode("reference")                   # no table to choose
+    plan.close()

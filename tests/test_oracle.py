@@ -383,3 +383,72 @@ def test_delayed_batch_correction_restores_the_clean_transform(dtype, Ni, n, BS,
     y[1, 0, :] += 100.0
     wrong = O.delayed_batch_correction(x, y, 0, n, dtype)
     assert O.rel_l2(wrong, clean[0]) > 100 * tol
+
+
+# ---- thread-level verification model ----
+
+@pytest.mark.parametrize("R", [2, 4, 8, 16, 32, 64])
+def test_thread_level_vectors_satisfy_the_checksum_identity(R):
+    # sum_o y_o r[o%3] == sum_i x_i c_R[i] for y = DFT_R(x), with the DFT taken by brute force: a
+    # transposed index, a conjugated root or r used on the input side breaks this by O(|x|)
+    rng = np.random.default_rng(R)
+    x = rng.normal(size=(5, R)) + 1j * rng.normal(size=(5, R))
+    y = O.dft_bruteforce(x)
+    cR, rR = O.thread_level_vectors(R, "double2")
+    assert np.allclose((y * rR).sum(axis=1), (x * cR).sum(axis=1), rtol=0, atol=1e-12 * R)
+    assert np.allclose(rR, O.checksum_r()[np.arange(R) % 3])
+    # and the input-side vector is the block-level one of the same length
+    assert np.allclose(cR, O.dft_checksum_vector(R, "double2"), atol=1e-13 * R) if R >= 2 else True
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+@pytest.mark.parametrize("logNi,BS,n", [(10, 2, 16), (7, 8, 8), (13, 1, 32), (4, 4, 4), (9, 2, 8)])
+def test_thread_level_model_clean_and_injected(dtype, logNi, BS, n):
+    Ni = 1 << logNi
+    rng = np.random.default_rng(logNi)
+    x = rng.uniform(-1, 1, (5, BS, Ni)) + 1j * rng.uniform(-1, 1, (5, BS, Ni))
+    flagged, verdicts, quiet = O.thread_level_model(x, n, dtype)
+    assert not flagged.any() and not verdicts
+    assert quiet < (1e-6 if dtype == "float2" else 1e-14)          # rounding only
+    # 100 on re of element m of one sub-FFT after the first pass's input sums moves every output of
+    # that thread's first register-level DFT by 100: exactly one thread of pass 0 objects, by the
+    # closed-form shift -100 * sum_{o<R}(re r + im r) of its radix; later passes see consistent data
+    m = min(Ni // n - 1, 3)
+    inj = O.Injection(2, BS - 1, m, 100.0)
+    flagged, verdicts, quiet = O.thread_level_model(x, n, dtype, [inj])
+    assert list(np.nonzero(flagged)[0]) == [2]
+    assert [(v.tile, v.s, v.q, v.thread) for v in verdicts] == [(2, BS - 1, 0, m)]
+    R0 = O.radix_passes(Ni, n)[0]
+    # (sign: the model's delta is in - out, the block-level one in + (-out): the same quantity)
+    assert abs(verdicts[0].delta - O.injected_delta_closed_form(R0, 100.0)) < (1e-3 if dtype == "float2" else 1e-10)
+    assert quiet < (1e-6 if dtype == "float2" else 1e-14)
+
+
+@pytest.mark.parametrize("dtype", ["float2", "double2"])
+def test_thread_level_model_sees_a_fault_in_any_pass(dtype):
+    # a fault on one output of one register-level DFT, in each pass in turn: the owner thread of that
+    # pass objects (x = rest mod Ni/n), nobody else, and the shift is the fault weighed with r[o % 3]
+    logNi, BS, n = 10, 2, 8
+    Ni, Tr = 1 << logNi, (1 << logNi) // n
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, (3, BS, Ni)) + 1j * rng.uniform(-1, 1, (3, BS, Ni))
+    passes = O.radix_passes(Ni, n)
+    r = O.checksum_r()
+    for q, R in enumerate(passes):
+        rest, o, val = 37 % (Ni // R), R - 1, 5.0 - 2.0j
+        flagged, verdicts, quiet = O.thread_level_model(x, n, dtype, out_faults=[(1, 1, q, rest, o, val)])
+        assert list(np.nonzero(flagged)[0]) == [1]
+        assert [(v.tile, v.s, v.q, v.thread) for v in verdicts] == [(1, 1, q, rest % Tr)]
+        w = val * r[o % 3]
+        assert abs(verdicts[0].delta + (w.real + w.imag)) < (1e-3 if dtype == "float2" else 1e-10)
+
+
+def test_thread_level_plan_model_covers_every_launch():
+    row = O.PlanRow.from_list([12, 2, 6, 6, 0, 16, 16, 0, 8, 8, 0])
+    rng = np.random.default_rng(8)
+    x = (rng.uniform(-1, 1, (4, 1 << 12)) + 1j * rng.uniform(-1, 1, (4, 1 << 12))).astype(np.complex128)
+    res, out = O.thread_level_plan_model(x, row, "double2", [O.Injection(5, 3, 2, 100.0)], inj_launch=0)
+    assert list(np.nonzero(res[0][0])[0]) == [5] and not res[1][0].any()
+    assert O.rel_l2(out, O.fft_ref(x)) < O.tolerance("double2", 12)
+    res, out = O.thread_level_plan_model(x, row, "double2", [O.Injection(9, 0, 0, 100.0)])
+    assert not res[0][0].any() and list(np.nonzero(res[1][0])[0]) == [9]

@@ -215,7 +215,8 @@ class TurboFFT:
         self.N = 1 << self.logN
         self.datatype = _datatype(datatype)
         self.cdtype = np.complex64 if self.datatype == FP32 else np.complex128
-        self.if_ft = int(bool(if_ft or if_err))
+        # if_ft: 1 checksums per group of thread_bs tiles, 2 thread-level verification (every tile on its own)
+        self.if_ft = int(if_ft) if int(if_ft) in (1, 2) else int(bool(if_ft or if_err))
         self.if_err = int(bool(if_err))
         self.thread_bs = int(thread_bs)
         self._h = lib().turbofft_plan_create(self.logN, self.datatype, self.if_ft, self.if_err, self.thread_bs,

@@ -91,8 +91,15 @@ class KernelSpec:
         self.BS = k.BS
         self.n = k.n
         self.kind = k.kind
-        self.ft = bool(k.ft)
+        self.ft = int(k.ft) in (1, 2)   # block-level two-sided checksums over a group of tiles
         self.dc = int(k.ft) == 2    # delayed batch correction: sums of the group's inputs and outputs per thread
+        # thread-level verification: every thread checks each register-level radix-R DFT it computes
+        # (sum_o y_o r[o%3] against sum_i x_i c_R[i], the two-sided checksum of abft.h:21-61 applied to
+        # the thread's own butterflies) pass by pass; no sums leave the thread, the block only agrees on
+        # whether any thread objected, and a tile that one did object to is recomputed before it is stored
+        self.tl = int(k.ft) == 3
+        if self.tl and (k.pf or k.xl or k.ck or k.inv):
+            raise ValueError(f"{k}: thread-level verification has no prefetching, cross-lane, compact-table or inverse flavour")
         self.ck16 = bool(k.ck)      # compact checksum table: one cotangent per element (half precision for fp32, single for fp64)
         if self.ck16 and (int(k.ft) != 1 or k.n % 2 or k.pf):
             raise ValueError(f"{k}: the compact checksum table is for recompute-correcting kernels without prefetch")
@@ -149,7 +156,7 @@ class KernelSpec:
                 self.pads.append(lds_model.choose_padding(self, x))
         self.lds_elems = max([self.phys_const(self.E - 1, p) + 1 for p in self.pads] + [1])
         self.red_off_bytes = (self.lds_elems * self.lds_esize + 15) // 16 * 16
-        self.lds_bytes = self.red_off_bytes + (3 * (self.threads // WAVE) * 8 if self.ft else 0)
+        self.lds_bytes = self.red_off_bytes + (3 * (self.threads // WAVE) * 8 if self.ft else 0) + (16 * 4 if self.tl else 0)
         # compact checksum words parked in LDS (ck = 3): W words per thread behind the reduction
         # slots, four to an access, access g of thread tx at [g * threads + tx]
         self.ck_lds = int(k.ck) == 3
@@ -360,8 +367,12 @@ class KernelEmitter:
         last = q == sp.npass - 1
         M = sp.Ni // sp.P[q]
         c(f"// pass {q}: radix {R}, {U} butterfl{'y' if U == 1 else 'ies'} per thread, sub-FFT length {M}")
+        if sp.tl:
+            self.emit_tl_input(c, q)
         for u in range(U):
             self.emit_radix(c, [u + U * i for i in range(R)])
+        if sp.tl:
+            self.emit_tl_output(c, q)
         if last:
             return
         lP = ilog2(sp.P[q])
@@ -383,6 +394,66 @@ class KernelEmitter:
             self.emit_apply_powers(c, R, pow2, targets)
             c.ind -= 1
             c("}")
+
+    # ---------- thread-level verification ----------
+    @staticmethod
+    def tl_vectors(R: int):
+        """Checksum vectors of a radix-R DFT: output side r[o % 3] (abft.h:22-28, with its float-rounded
+        sqrt(3)/2) and input side c_R[i] = sum_o r[o % 3] W_R^(i o) (abft.h:45-60 with exact angles), each
+        as the pair (re + im, re - im) that makes re+im of a product two multiply-adds."""
+        s3 = 0.8660253882408142
+        r = [complex(1.0, 0.0), complex(-0.5, -s3), complex(-0.5, s3)]
+        cin = []
+        for i in range(R):
+            acc = 0j
+            for o in range(R):
+                ang = -2.0 * math.pi * ((i * o) % R) / R
+                acc += r[o % 3] * complex(math.cos(ang), math.sin(ang))
+            cin.append((acc.real + acc.imag, acc.real - acc.imag))
+        rout = [(v.real + v.imag, v.real - v.imag) for v in r]
+        return cin, rout
+
+    def emit_tl_input(self, c: Code, q: int):
+        """Before the butterflies of pass q: the thread's input-side sum over its U radix-R DFTs, then
+        (first pass only) the compute-side error injection of fft_codegen.py:412-415."""
+        sp = self.s
+        R = sp.passes[q]
+        U = sp.n // R
+        cin, _ = self.tl_vectors(R)
+        c(f"{self.R} tin = 0, tiy = 0, tout = 0, toy = 0;")
+        c("if (!is_redo) {")
+        c.ind += 1
+        for u in range(U):
+            for i in range(R):
+                reg = u + U * i
+                c(f"tin += r[{reg}].x * {self.lit(cin[i][0])}; tiy += r[{reg}].y * {self.lit(cin[i][1])};")
+        if q == 0:
+            # the injected element is one of the first Ni/n of its sub-FFT (register 0 of thread x = m;
+            # the reference injects at m = 0), after the input-side sum has been taken
+            c(f"r[0].x += (inj_hit && s == (unsigned)a.ft.inj_s && x == (unsigned)a.ft.inj_m) ? ({self.R})a.ft.inj_mag : ({self.R})0;")
+        c.ind -= 1
+        c("}")
+
+    def emit_tl_output(self, c: Code, q: int):
+        """After the butterflies of pass q and before its twiddles: the output-side sum and the thread's
+        own verdict, |in - out| / (err_smoothing + |in| + |out|) > err_threshold (the rule of
+        fft_codegen.py:495 on this thread's two sums)."""
+        sp = self.s
+        R = sp.passes[q]
+        U = sp.n // R
+        lR = ilog2(R)
+        _, rout = self.tl_vectors(R)
+        c("if (!is_redo) {")
+        c.ind += 1
+        for u in range(U):
+            for o in range(R):
+                reg = u + U * bitrev(o, lR)
+                c(f"tout += r[{reg}].x * {self.lit(rout[o % 3][0])}; toy += r[{reg}].y * {self.lit(rout[o % 3][1])};")
+        c(f"const {self.R} ti = tin + tiy, to = tout + toy;")
+        c(f"if (fabs(ti - to) / (({self.R})a.ft.err_smoothing + fabs(ti) + fabs(to)) > ({self.R})a.ft.err_threshold) tbad = true;")
+        c.ind -= 1
+        c("}")
+        c("(void)tin; (void)tiy; (void)tout; (void)toy;")
 
     def emit_lds_write(self, c: Code, q: int, part: str = ""):
         """Store the outputs of pass q in the layout pass q+1 reads
@@ -886,6 +957,8 @@ class KernelEmitter:
             c = Code()
             self.map_vars(c, q)
             c(f"{self.T2} t;")
+            if q == 0 and sp.tl:
+                c("tbad = false;")
             if q == 0 and sp.pfk:
                 # the first pfk elements were fetched during the previous tile's last pass
                 for e in range(sp.pfk):
@@ -966,6 +1039,24 @@ class KernelEmitter:
                     continue
                 if sp.ft:
                     self.emit_ft_output(c)
+                if sp.tl:
+                    # The tile waits in registers for the block's verdict: every wavefront leaves a word that
+                    # says whether one of its threads objected, the block reads them all behind a barrier
+                    # (separator "vote", emitted by emit()), and only an accepted tile -- or the recomputed
+                    # one -- is stored.
+                    c("(void)t;")
+                    c(f"TL_VOTE({sp.red_off_bytes + (3 * (sp.threads // WAVE) * 8 if sp.ft else 0)}, tbad);")
+                    out.append(("barrier", c.text()))
+                    st = Code()
+                    self.map_vars(st, q)
+                    st("(void)x; (void)s;")
+                    st("if (is_redo || !(tany && a.ft.correct)) {")
+                    st.ind += 1
+                    self.emit_store(st)
+                    st.ind -= 1
+                    st("}")
+                    out.append(("vote", st.text()))
+                    continue
                 if sp.dc:
                     # the only tile of a group is held back until the group has been checked
                     c("if (!hold || is_redo) {")
@@ -1005,7 +1096,7 @@ class KernelEmitter:
         c = Code()
         T2, R = self.T2, self.R
         c(f"// {sp.name}: {sp.kind} kernel, {T2}, Ni={sp.Ni}, BS={sp.BS}, n={sp.n}, passes={'x'.join(map(str, sp.passes))},")
-        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}{', cross-lane last pass' if sp.xl else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' + (' (delayed batch correction)' if sp.dc else '') if sp.ft else ''}")
+        c(f"// {sp.threads} threads, LDS {sp.lds_bytes} B{' (split re/im exchange)' if sp.split else ''}{', next-tile prefetch' if sp.pf else ''}{', cross-lane last pass' if sp.xl else ''}, thread maps {sp.maps}, pads {sp.pads}{', fault tolerant' + (' (delayed batch correction)' if sp.dc else '') if sp.ft else ''}{', thread-level verification' if sp.tl else ''}")
         if sim:
             c(f'extern "C" void {sp.name}_sim(const {T2}* in, {T2}* out, const {T2}* tw, const tfft_kargs* ap, long long grid, const long long* limits)')
             c("{")
@@ -1015,7 +1106,7 @@ class KernelEmitter:
             c("const long long twhi_limit = limits[3], twlo_limit = limits[4], ck_limit = limits[5];")
             c(f"const long long lds_limit = {sp.lds_elems};")
             c("(void)in_limit; (void)out_limit; (void)tw_limit; (void)twhi_limit; (void)twlo_limit; (void)ck_limit; (void)lds_limit;")
-            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; unsigned cwr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; }};")
+            c(f"struct TS {{ {T2} r[{sp.n}]; {T2} rn[{sp.n}]; {T2} sh[{sp.n}]; {T2} cvr[{sp.n}]; unsigned cwr[{sp.n}]; {T2} sx[{sp.n}]; {T2} sy[{sp.n}]; {R} fin1, fin2, fo1, fo2; bool tbad; }};")
             c("for (long long pbx = 0; pbx < grid; ++pbx) {")
             c.ind += 1
             c("long long bx = pbx; const long long pbx_raw = pbx; (void)pbx_raw;")
@@ -1038,6 +1129,8 @@ class KernelEmitter:
             c(f"{T2} r[{sp.n}];")
             if sp.pf:
                 c(f"{T2} rn[{sp.pfk or sp.n}];")
+            if sp.tl:
+                c("bool tbad = false;")
             if sp.ft:
                 c(f"{R} fin1 = 0, fin2 = 0, fo1 = 0, fo2 = 0;")
                 if self.ft_table_resident():
@@ -1125,6 +1218,23 @@ class KernelEmitter:
             c("if (a.ft.inj_mode == 1) inj_hit = (it == (int)(bx % a.thread_bs)) && (bx % a.ft.inj_every == 0);")
             c("else if (a.ft.inj_mode == 2) inj_hit = (tile % a.ft.inj_every) == a.ft.inj_tile;")
             c("(void)cntf; (void)inj_hit;")
+        elif sp.tl:
+            # tiles checked: one per tile, counted once per launch by its first block
+            if sim:
+                c("if (pbx == 0) a.ft.counters[0] += (unsigned long long)a.ntiles;")
+            else:
+                c("if (blockIdx.x == 0 && tx == 0) atomicAdd(&a.ft.counters[0], (unsigned long long)a.ntiles);")
+            c("for (int it = it0; it < it1; ++it) {")
+            c.ind += 1
+            c("const long long tile = tile0 + it * gstride;")
+            c("bool inj_hit = false;")
+            c("if (a.ft.inj_mode == 1) inj_hit = (it == (int)(bx % a.thread_bs)) && (bx % a.ft.inj_every == 0);")
+            c("else if (a.ft.inj_mode == 2) inj_hit = (tile % a.ft.inj_every) == a.ft.inj_tile;")
+            c("(void)inj_hit;")
+            # second trip: the tile is transformed again, unchecked, when a thread objected to the first
+            c("for (int trip = 0; trip < 2; ++trip) {")
+            c.ind += 1
+            c("const bool is_redo = trip != 0;")
         else:
             c("for (int it = it0; it < it1; ++it) {")
             c.ind += 1
@@ -1139,8 +1249,10 @@ class KernelEmitter:
             if i:
                 if sim:
                     c(f"// ---- {sep} ----")
-                elif sep == "barrier":
+                elif sep in ("barrier", "vote"):
                     c("__syncthreads();")
+            if sep == "vote":
+                self.emit_tl_verdict(c, sim)
             self.thread_block(c, sim, ph)
         if sp.ft:
             self.emit_ft_decide(c, sim)
@@ -1165,6 +1277,10 @@ class KernelEmitter:
                 self.thread_block(c, sim, pre.text())
                 c.ind -= 1
                 c("}")
+        if sp.tl:
+            c("if (is_redo || !(tany && a.ft.correct)) break;")
+            c.ind -= 1
+            c("}")  # trip loop
         c.ind -= 1
         c("}")  # tile loop
         if parts:
@@ -1191,12 +1307,38 @@ class KernelEmitter:
         if sim:
             c(f"for (unsigned tx = 0; tx < {sp.threads}u; ++tx) {{")
             c.ind += 1
-            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& cwr = ts[tx].cwr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2;")
-            c("(void)r; (void)rn; (void)cvr; (void)cwr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2;")
+            c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& cwr = ts[tx].cwr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2; auto& tbad = ts[tx].tbad;")
+            c("(void)r; (void)rn; (void)cvr; (void)cwr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2; (void)tbad;")
         else:
             c("{")
             c.ind += 1
         c(body.rstrip("\n"))
+        c.ind -= 1
+        c("}")
+
+    def emit_tl_verdict(self, c: Code, sim: bool):
+        """Thread-level verification, behind the barrier that follows a tile's last pass: did any thread of the
+        block object?  A detection is counted and listed like one of the block-level scheme (one atomic on
+        one of 64 counter lines); the tile is its own group, so it needs no locating."""
+        sp = self.s
+        nw = sp.threads // WAVE
+        off = sp.red_off_bytes + (3 * nw * 8 if sp.ft else 0)
+        if sim:
+            c("bool tany = false; for (auto& z : ts) tany = tany || z.tbad;")
+            c("if (tany && !is_redo) {")
+        else:
+            c("bool tany = false;")
+            c(f"{{ const unsigned* tv = (const unsigned*)(lds_raw + {off}); unsigned tor = 0u; for (int w = 0; w < {nw}; ++w) tor |= tv[w]; tany = tfft_uni(tor) != 0u; }}")
+            if sp.npass_lds < 2:
+                # no other barrier separates this read from the next trip's votes
+                c("__syncthreads();")
+            c("if (tany && !is_redo && tx == 0) {")
+        c.ind += 1
+        c("const unsigned sub = (unsigned)(pbx_raw & 63);")
+        c("unsigned long long* sc = a.ft.counters + TFFT_FT_SUB0 + TFFT_FT_SUB_STRIDE * sub;")
+        c("const unsigned long long region = (unsigned long long)(a.ft.flagged_cap >> 6);")
+        c("const unsigned long long slot = sc[0]++;" if sim else "const unsigned long long slot = atomicAdd(sc, 1ull);")
+        c("if (slot < region) { long long* fl = a.ft.flagged + 2 * (sub * region + slot); fl[0] = a.ft.launch; fl[1] = tile; }")
         c.ind -= 1
         c("}")
 

@@ -80,7 +80,10 @@ class KernelKey:
     n: int
     ft: int          # 0 plain; 1 fused checksums, a located tile is recomputed from its input; 2 the same
                      # checksums with delayed batch correction (per-thread sums of the group's inputs and
-                     # outputs, the located tile is patched with FFT(sum x) - sum y)
+                     # outputs, the located tile is patched with FFT(sum x) - sum y); 3 thread-level
+                     # verification: every thread checks the register-level DFTs it computes in each pass
+                     # against the checksum vector of their radix, no block-wide sums, a flagged tile is
+                     # recomputed before it is stored
     split: int = 0   # 1: every LDS exchange moves re and im in two rounds through a half-size buffer
     pf: int = 0      # 1: the next tile is fetched into a second register set while this one is computed;
                      # k > 1: only the first k elements of a thread, from the start of the tile's last pass on
@@ -99,7 +102,7 @@ class KernelKey:
     def name(self) -> str:
         t = "f32" if self.dtype == "float2" else "f64"
         return (f"tfft_{t}_{self.kind}_N{self.logNi}_b{self.BS}_n{self.n}" + ("_s" if self.split else "") + ("_p" if self.pf == 1 else (f"_p{self.pf}" if self.pf else "")) + ("_x" if self.xl else "")
-                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2", 3: "_h3"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd"}[int(self.ft)]))
+                + (f"_w{self.wv}" if self.wv else "") + (f"_t{self.nt}" if self.nt else "") + ("_i" if self.inv else "") + ({0: "", 1: "_h", 2: "_h2", 3: "_h3"}[int(self.ck)]) + ({0: "", 1: "_ft", 2: "_fd", 3: "_tt"}[int(self.ft)]))
 
 
 def load_plan_csv(path: str) -> List[PlanRow]:
@@ -127,13 +130,15 @@ def kernels_for_row(row: PlanRow, dtype: str, ft: int, inverse: bool = False, co
     last = row.launches - 1
     return [KernelKey(dtype, kind, row.logNi[i], row.BS[i], row.n[i], int(ft), int(row.split[i]) if row.split else 0,
                       # (partial prefetch, pf > 1, exists for the plain forward kernel only)
-                      (int(row.pf[i]) if (int(row.pf[i]) <= 1 or not (ft or (inverse and i in (0, last)))) else 0) if row.pf else 0,
+                      ((int(row.pf[i]) if (int(row.pf[i]) <= 1 or not (ft or (inverse and i in (0, last)))) else 0) if row.pf else 0) if int(ft) != 3 else 0,
                       # fault-tolerant plans keep the LDS path: the checksum model fixes which
                       # outputs a thread owns
                       (int(row.xl[i]) if row.xl else 0) if not ft else 0,
                       # the register budget hint was tuned on the plain kernel only (fault-tolerant
                       # kernels keep their table in registers and spill under any tighter budget)
                       # (the compact-table flavour is the exception: its budget is tuned with it)
+                      # (thread-level verification runs the plain rows without their hint: timed with budgets of 2, 3 and
+                      # none for every size, none was the best or within a point of it at all but two)
                       (int(row.wv[i]) if row.wv else 0) if (not ft or (compact and int(ft) == 1 and row.ck and int(row.ck[i]))) else 0,
                       # the priority bit was timed on the plain kernel only
                       (int(row.nt[i]) & (3 if ft else 7)) if row.nt else 0,

@@ -134,6 +134,9 @@ __device__ __forceinline__ long long tfft_uni(long long v) {
 }
 // instruction-scheduling fence: nothing may be moved across it
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// thread-level verification: one word per wavefront at byte `off` of the block's LDS says whether any of
+// its lanes objected to the tile (a wave vote, then lane 0 writes); the block reads the words behind a barrier
+#define TL_VOTE(off, bad) { const int wany_ = __any((bad) ? 1 : 0); if ((tx & 63u) == 0u) ((unsigned*)(lds_raw + (off)))[tx >> 6] = wany_ ? 1u : 0u; }
 #else
 #include <cmath>
 #include <cstdio>
@@ -171,6 +174,7 @@ extern long long tfft_sim_errors;
 #define OPAQUE(v)
 template <typename T> static inline T tfft_uni(T v) { return v; }
 #define SCHED_FENCE()
+#define TL_VOTE(off, bad) ((void)0)
 // compact checksum table (ck_limit counts complex elements of the buffer the launcher passed)
 #define CKW(p, c, i) (((const unsigned*)(p))[TFFT_CHK((long long)(c) + (long long)(i), (long long)(sizeof(*(p)) / 4) * ck_limit, "compact checksum table")])
 static inline float tfft_ckh(unsigned w, int hi) {

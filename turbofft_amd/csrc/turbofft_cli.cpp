@@ -46,6 +46,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
     bool param_given = false;        // --param names the CSV; otherwise --gpu selects it
     bool if_sync = false;            // also print the reference's sync-after-every-launch timing
     int ft_correction = 1;           // 1 recompute the located tile, 2 delayed batch correction
+    int ft_scheme = 0;               // 0 checksums per group of tiles (the reference's current generator), 1 thread-level verification
 
     static void displayHelp() {
         std::cout << "Usage: program [options]\n"
@@ -68,6 +69,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
                   << "  --param <file>       Plan CSV (overrides the one --gpu selects).\n"
                   << "  --if_sync <0|1>      Also time with a host wait after every launch, as the reference does.\n"
                   << "  --ft_correction <1|2> With --if_err: recompute the located tile (1) or delayed batch correction (2).\n"
+                  << "  --ft_scheme <0|1>    With --if_ft: checksums per group of tiles (0) or thread-level verification (1).\n"
                   << "  --logN_begin/--logN_end <value>  Restrict the --if_bench sweep.\n"
                   << "  --param_1 <value>        logBS + logN of the --if_bench sweep (default 28; the reference derives it from --gpu).\n"
                   << "  -h, --help               Display this help message and exit.\n";
@@ -89,6 +91,7 @@ struct ProgramConfig {           // CommandLineParser.h:4-25
         else if (!strcmp(name, "--param")) { param_file_path = value; param_given = true; }
         else if (!strcmp(name, "--if_sync")) if_sync = atol(value);
         else if (!strcmp(name, "--ft_correction")) ft_correction = atoi(value);
+        else if (!strcmp(name, "--ft_scheme")) ft_scheme = atoi(value);
         else if (!strcmp(name, "--logN_begin")) logN_begin = atoi(value);
         else if (!strcmp(name, "--logN_end")) logN_end = atoi(value);
         else if (!strcmp(name, "--param_1")) { param_1 = atoi(value); param_1_given = true; }
@@ -225,7 +228,7 @@ int initializeData(Buffers& b, int datatype, long long points, bool fill) {
 // test_turbofft (main.cu:4-73): warm-up, ntest timed runs, the metric line
 int test_turbofft(const ProgramConfig& cfg, int logN, long long bs, int ntest, Buffers& b, std::vector<char>* result) {
     const char* csv = cfg.param_file_path.empty() ? nullptr : cfg.param_file_path.c_str();
-    turbofft_plan_t* plan = turbofft_plan_create(logN, cfg.datatype, cfg.if_ft, cfg.if_err, cfg.thread_bs, csv);
+    turbofft_plan_t* plan = turbofft_plan_create(logN, cfg.datatype, (cfg.if_ft && cfg.ft_scheme == 1) ? 2 : (int)cfg.if_ft, cfg.if_err, cfg.thread_bs, csv);
     if (!plan) { printf("turboFFT, %d: %s\n", logN, turbofft_last_error()); return -1; }
     float ms = 0;
     int rc = TURBOFFT_OK;

@@ -211,6 +211,7 @@ struct c64 { double x, y; };
 
 struct turbofft_plan {
     int logN = 0, datatype = 0, if_ft = 0, if_err = 0, thread_bs = 1;
+    int scheme = 0;                // fault-tolerant plans: 0 block-level two-sided checksums over a group of tiles, 1 thread-level verification
     bool tiles_from_row = false;   // thread_bs is the plan row's tuned tiles-per-block, not the caller's
     Row row{};
     int launches = 0;
@@ -400,7 +401,7 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
     } else {
         std::istringstream in(tfft_builtin_param_csv(p->datatype));
         if (!parse_csv(in, rows)) return fail(TURBOFFT_ENOPLAN, "built-in plan table is malformed");
-        if (p->if_ft) {
+        if (p->if_ft && p->scheme == 0) {
             // the checksum flavour of a kernel needs more registers: where another tile shape
             // measured faster with checksums, the built-in table carries a replacement row
             std::istringstream fin(tfft_builtin_param_ft_csv(p->datatype));
@@ -474,14 +475,17 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
     long long twN = 1;
     for (int i = 0; i < p->launches; ++i) {
         int kind = kind_of_launch(p->launches, i);
-        const tfft_kernel_entry* k = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, (p->if_ft && r.pf(i) > 1) ? 0 : r.pf(i),
+        const tfft_kernel_entry* k = p->scheme == 1
+            // thread-level verification runs the plain rows: same shape, exchange form and cache policy, no register budget hint
+            ? find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 3, r.split(i) ? 1 : 0, 0, 0, 0, r.nt(i) & 3)
+            : find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i) ? 1 : 0, (p->if_ft && r.pf(i) > 1) ? 0 : r.pf(i),
                                                  (r.xl(i) && !p->if_ft) ? 1 : 0,    // FT plans keep the LDS path
                                                  p->if_ft ? 0 : r.wv(i), p->if_ft ? (r.nt(i) & 3) : r.nt(i));   // wave budget and priority bit: plain kernels only
         if (!k)
             return fail(TURBOFFT_ENOPLAN, "no compiled kernel for launch %d of logN=%d (type %d kind %d logNi %d BS %d n %d ft %d split %d prefetch %d)",
                         i, p->logN, p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), p->if_ft, r.split(i), r.pf(i));
         p->k_full[i] = k;
-        if (p->if_ft && r.ck(i)) {
+        if (p->if_ft && p->scheme == 0 && r.ck(i)) {
             // the row asks for the flavour that reads the compact checksum table; the full-table
             // flavour stays available for the table modes and thresholds the compact form cannot serve
             const tfft_kernel_entry* kc = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 1, r.split(i) ? 1 : 0, 0, 0, r.wv(i), r.nt(i) & 3, 0, r.ck(i));
@@ -493,7 +497,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
             k = kc;
         }
         p->k[i] = k;
-        if (p->if_ft) {
+        if (p->if_ft && p->scheme == 0) {
             p->k_dc[i] = find_kernel(p->datatype, kind, r.logNi(i), r.BS(i), r.n(i), 2, r.split(i) ? 1 : 0, 0, 0, 0, r.nt(i) & 3);
             if (p->k_dc[i] && p->k_dc[i]->lds_bytes > kCuLdsBytes) p->k_dc[i] = nullptr;   // no such flavour on this device
             if (p->k_dc[i]) if (int rc = allow_lds(p->k_dc[i], prop)) return rc;
@@ -561,7 +565,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
             HIP_TRY(hipMemcpy(p->tw_lo[i], host.data(), host.size(), hipMemcpyHostToDevice));
         }
     }
-    if (p->if_ft) {
+    if (p->if_ft && p->scheme == 0) {
         for (int i = 0; i < p->launches; ++i)
             HIP_TRY(hipMalloc(&p->cksum[i], ((size_t)1 << r.logNi(i)) * p->esize));
         int rc = upload_checksum_tables(p);
@@ -583,7 +587,7 @@ static int plan_build_row(turbofft_plan* p, const Row& row) {
         // overlap that block scheduling provides, and few long groups leave CUs idle.
         int part_len = kPartLen;
         if (const char* e = getenv("TURBOFFT_FT_PART_LEN")) part_len = atoi(e);
-        if (part_len > 0 && p->thread_bs > part_len) {
+        if (part_len > 0 && p->thread_bs > part_len && p->scheme == 0) {
             // (a plan row may name its own length per launch, columns 34-36 of the fault-tolerant table; groups of up to
             // kPartLen tiles are never shared, whatever the row says: sharing them measured slower at most sizes)
             for (int i = 0; i < p->launches; ++i) p->ft_part_len[i] = (p->row.gp(i) > 0 && !getenv("TURBOFFT_FT_PART_LEN")) ? p->row.gp(i) : part_len;
@@ -598,11 +602,13 @@ turbofft_plan_t* turbofft_plan_create(int logN, int datatype, int if_ft, int if_
     g_err.clear();
     if (datatype != TURBOFFT_FP32 && datatype != TURBOFFT_FP64) { fail(TURBOFFT_EINVAL, "bad datatype %d", datatype); return nullptr; }
     if (thread_bs < 1) { fail(TURBOFFT_EINVAL, "thread_bs must be >= 1"); return nullptr; }
+    if (if_ft < 0 || if_ft > 2) { fail(TURBOFFT_EINVAL, "if_ft must be 0 (none), 1 (checksums per group of tiles) or 2 (thread-level verification)"); return nullptr; }
     turbofft_plan* p = new turbofft_plan();
     p->logN = logN;
     p->datatype = datatype;
     p->if_err = if_err ? 1 : 0;
     p->if_ft = (if_ft || if_err) ? 1 : 0;            // CommandLineParser.h:66-68
+    p->scheme = if_ft == 2 ? 1 : 0;
     p->thread_bs = thread_bs;
     if (p->if_err) { p->inj_mode = 1; p->correct = 1; }   // the if_err=1 kernels inject and correct
     const char* env = getenv("TURBOFFT_CHECKSUM_MODE");
@@ -685,6 +691,7 @@ int turbofft_set_ft_params(turbofft_plan_t* p, double err_smoothing, double err_
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
     if (correct < 0 || correct > 2) return fail(TURBOFFT_EINVAL, "correct must be 0 (detect only), 1 (recompute) or 2 (delayed batch correction)");
+    if (correct == 2 && p->scheme == 1) return fail(TURBOFFT_EINVAL, "thread-level verification recomputes a flagged tile before it is stored: correct is 0 or 1");
     if (correct == 2)
         for (int i = 0; i < p->launches; ++i)
             if (!p->k_dc[i])
@@ -802,6 +809,7 @@ int turbofft_set_checksum_mode(turbofft_plan_t* p, int mode) {
     if (!p) return fail(TURBOFFT_EINVAL, "null plan");
     if (!p->if_ft) return fail(TURBOFFT_EINVAL, "plan was created without if_ft");
     if (mode != 0 && mode != 1) return fail(TURBOFFT_EINVAL, "checksum mode must be 0 (exact) or 1 (reference)");
+    if (p->scheme == 1) return fail(TURBOFFT_EINVAL, "thread-level verification reads no checksum table (its vectors are constants of the kernels)");
     hipStream_t st = nullptr;
     int rc = sync_last_stream(p, &st);      // executions in flight still read the old tables
     if (rc) return rc;
@@ -1045,7 +1053,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.logQ = p->launches == 3 ? r.logNi(1) : 0;
         }
         if (p->if_ft) {
-            a.ft.cksum = k->ck ? p->cksum16[i] : p->cksum[i];
+            a.ft.cksum = p->scheme == 1 ? nullptr : (k->ck ? p->cksum16[i] : p->cksum[i]);
             a.ft.counters = p->counters;
             a.ft.flagged = p->flagged;
             a.ft.flagged_cap = p->flagged_cap;
