@@ -323,6 +323,9 @@ def main():
     ap.add_argument("--membench", action="store_true",
                     help="time the streaming yardsticks (copy with 8- and 16-byte lanes, read only, write only) "
                          "on 2 GiB and print one JSON line")
+    ap.add_argument("--membench_fused", type=str, default=None, metavar="G:R:B",
+                    help="--membench: only the two-pass copy through a per-XCD ring of R slots of G 512 KiB pieces with B blocks per CU "
+                         "(for counter runs of one configuration)")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -344,15 +347,46 @@ def main():
         for _ in range(20):
             turbofft_amd.membench(0, src.data_ptr(), dst.data_ptr(), nbytes, 0, 10, st)      # clock the device up
         res = {}
+        only_fused = [tuple(int(t) for t in a.membench_fused.split(":"))] if a.membench_fused else None
         # every kernel plain, then with what the FFT kernels use: non-temporal accesses (+4), XCD-aware
         # tile order (+8) and a bound on the blocks resident per CU (+16*k; the exchange buffer of an
         # FFT kernel bounds it to 2-4)
         flavours = (("", 0), ("_nt", 4), ("_nt_xcd", 12), ("_nt_xcd_2percu", 12 + 32), ("_nt_xcd_3percu", 12 + 48), ("_nt_xcd_4percu", 12 + 64), ("_nt_xcd_6percu", 12 + 96))
         for kind, name, moved in ((0, "copy_8B_lanes", 2), (1, "copy_16B_lanes", 2), (2, "read_only", 1), (3, "write_only", 1)):
+            if only_fused:
+                break
             for sfx, bits in flavours:
                 ms = sorted(turbofft_amd.membench(kind + bits, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))
                 res[name + sfx] = {"ms_per_pass_median": ms[2], "ms_min": ms[0], "ms_max": ms[4], "GB/s": moved * nbytes / ms[2] / 1e6}
                 print(f"{name + sfx:32s} {ms[2]:.4f} ms  {moved * nbytes / ms[2] / 1e6:7.0f} GB/s", file=sys.stderr, flush=True)
+        # the access patterns of the column kernels and of the transposed store: runs of 128-512 bytes at a large stride
+        strided = {}
+        for ls in (() if only_fused else (12, 14, 16, 19)):
+            for run in (128, 256, 512):
+                for lane in (8, 16):
+                    for write in (0, 1):
+                        best = None
+                        for xc in (4, 16, 64):
+                            ms = sorted(turbofft_amd.membench_strided(write, lane, run, ls, xc, src.data_ptr(), dst.data_ptr(), nbytes, 3, 10, st) for _ in range(3))[1]
+                            if best is None or ms < best[0]:
+                                best = (ms, xc)
+                        name = f"{'write' if write else 'read'}_run{run}_stride2^{ls}_{lane}B_lanes"
+                        strided[name] = {"ms_per_pass": best[0], "GB/s": nbytes / best[0] / 1e6, "tiles_per_xcd_run": best[1]}
+                        print(f"{name:40s} {best[0]:.4f} ms  {nbytes / best[0] / 1e6:7.0f} GB/s  (runs of {best[1]} tiles per XCD)", file=sys.stderr, flush=True)
+        res["strided"] = strided
+        # two passes through a ring meant to stay in the XCD's L2, against two whole passes
+        scratch = torch.empty((8 * 3 * 8 * 512 * 1024) // 4, device="cuda", dtype=torch.float32)
+        fused = {}
+        two = sorted(turbofft_amd.membench(12, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))[2] * 2
+        fused["two_whole_passes_ms"] = two
+        for G, R, bpc in (only_fused or ((1, 3, 2), (2, 3, 2), (4, 2, 2), (4, 3, 2), (8, 3, 2), (8, 3, 3))):
+            dst.zero_()
+            ms, stt = turbofft_amd.membench_fused(G, R, bpc, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, 50, 1, 5, st)
+            ok = bool(torch.equal(src, dst))
+            fused[f"group{G}_slots{R}_blocks{bpc}"] = {"ms": ms, "ring_KiB_per_xcd": G * R * 512, "copied_right": ok, **stt}
+            print(f"fused copy: {G} x 512 KiB per group, {R} slots ({G * R * 512} KiB ring per XCD), {bpc} blocks per CU: {ms:.3f} ms "
+                  f"(two whole passes {two:.3f} ms), right {ok}, {stt}", file=sys.stderr, flush=True)
+        res["fused_two_pass_copy"] = fused
         print(json.dumps({"membench": res, "bytes": nbytes, "tile_bytes": 65536, "threads": 256}), flush=True)
         return 0
     if a.sweep:

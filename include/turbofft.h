@@ -345,6 +345,27 @@ int turbofft_offline_ft_time(int logN, int datatype, const void* in_d, void* out
 int turbofft_membench(int mode, const void* src_d, void* dst_d, size_t bytes, int warmup, int reps,
                       void* stream, float* ms_per_pass);
 
+/* Read-only (write = 0: sweeps src) or write-only (write = 1: fills dst) pass over `bytes` in 64 KiB tiles that
+ * are rows of `run_bytes` (128, 256, 512) at a stride of 2^log_stride bytes -- the access pattern of the column
+ * kernels (runs of BS elements at the stride of their digit) and of the transposed store of the last launch --
+ * with lanes of `lane_bytes` (8, 16), non-temporal accesses and runs of `xcd_chunk` consecutive tiles per XCD
+ * (0: plain block order).  `bytes` is a multiple of (65536 / run_bytes) << log_stride. */
+int turbofft_membench_strided(int write, int lane_bytes, int run_bytes, int log_stride, int xcd_chunk, const void* src_d,
+                              void* dst_d, size_t bytes, int warmup, int reps, void* stream, float* ms_per_pass);
+
+/* Two passes through a ring that is meant to stay in the XCD's L2: a copy src -> ring -> dst as ONE persistent
+ * kernel (`blocks_per_cu` blocks per CU), the data cut into 512 KiB pieces that the 8 XCDs own in turn, each XCD
+ * with `ring_slots` (2..8) slots of `group` pieces inside `scratch_d` (8 * ring_slots * group * 512 KiB), reused for
+ * every group; the second pass of a group starts when its first pass is complete, as the row pass of a two-launch
+ * plan needs every column tile of its transform.  Measures whether a fused pass pair could keep its intermediate
+ * on chip (rocprofv3's FETCH_SIZE / WRITE_SIZE of the kernel tell where the ring's traffic went).  Every wait inside
+ * the kernel is for work that running blocks hold and is bounded by `limit_ms` per launch: on a time-out the kernel
+ * drains and stats[0] is 1.  stats: [0] time-out flag, [1] waits that had to poll, [2] polls, [3] blocks launched,
+ * [4..11] blocks that ran on each XCD.  dst equals src afterwards.  `bytes` is a multiple of 4 MiB. */
+int turbofft_membench_fused(int group, int ring_slots, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+                            void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
+                            unsigned stats[12]);
+
 /* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
  * flags and output lines.  Returns the process exit code. */
 int turbofft_main(int argc, char** argv);

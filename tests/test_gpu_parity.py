@@ -810,3 +810,41 @@ def test_exec_inside_a_hip_graph(dt, logN, bs, ft):
         else:
             assert c["detected"] == 0
     plan.close()
+
+
+def test_streaming_yardsticks_run():
+    # the measurement kernels of known traffic (nothing of a transform): every flavour moves what it says,
+    # the fused two-pass copy through the per-XCD ring copies right and never runs into its time limit
+    torch = _torch()
+    nbytes = 256 << 20
+    src = torch.rand(nbytes // 4, device="cuda", dtype=torch.float32)
+    dst = torch.zeros(nbytes // 4, device="cuda", dtype=torch.float32)
+    st = torch.cuda.current_stream().cuda_stream
+    for mode in (0, 1, 4, 5, 12, 13, 12 + 48):
+        dst.zero_()
+        assert turbofft_amd.membench(mode, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st) > 0
+        assert torch.equal(src, dst)
+    assert turbofft_amd.membench(2 + 12, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st) > 0
+    assert turbofft_amd.membench(3 + 12, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st) > 0
+    for lane in (8, 16):
+        for run in (128, 256, 512):
+            for ls in (12, 19):
+                keep = src.clone()
+                assert turbofft_amd.membench_strided(False, lane, run, ls, 16, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st) > 0
+                assert torch.equal(src, keep)
+                dst.zero_()
+                assert turbofft_amd.membench_strided(True, lane, run, ls, 4, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st) > 0
+                v = dst.view(-1, 2)
+                assert bool((v[:, 1] == 1).all())              # every 8-byte element of the buffer was written
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        turbofft_amd.membench_strided(True, 8, 100, 12, 4, src.data_ptr(), dst.data_ptr(), nbytes, 1, 2, st)
+    scratch = torch.empty((8 * 3 * 2 * 512 * 1024) // 4, device="cuda", dtype=torch.float32)
+    for G, R, bpc in ((1, 2, 2), (2, 3, 3), (1, 3, 8)):
+        dst.zero_()
+        ms, stats = turbofft_amd.membench_fused(G, R, bpc, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, 200, 1, 2, st)
+        assert ms > 0 and stats["timed_out"] == 0 and sum(stats["blocks_per_xcd"]) == stats["blocks"]
+        assert torch.equal(src, dst)
+    with pytest.raises(turbofft_amd.TurboFFTError):           # the ring does not fit the scratch buffer
+        turbofft_amd.membench_fused(4, 3, 2, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes)
+    with pytest.raises(turbofft_amd.TurboFFTError):           # one slot: a first pass would wait for a later ticket
+        turbofft_amd.membench_fused(1, 1, 2, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes)

@@ -96,6 +96,8 @@ def lib() -> C.CDLL:
     L.turbofft_vendor_exec.argtypes = [i, i, vp, vp, ll, vp]
     L.turbofft_vendor_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_membench.argtypes = [i, vp, vp, C.c_size_t, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_membench_strided.argtypes = [i, i, i, i, i, vp, vp, C.c_size_t, i, i, vp, C.POINTER(C.c_float)]
+    L.turbofft_membench_fused.argtypes = [i, i, i, vp, vp, C.c_size_t, vp, C.c_size_t, i, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_uint)]
     L.turbofft_offline_checksums.argtypes = [i, i, vp, vp, ll, vp, vp, vp]
     L.turbofft_offline_ft_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_ulonglong)]
     _lib = L
@@ -188,6 +190,25 @@ def offline_ft_time(logN: int, datatype, in_ptr: int, out_ptr: int, bs: int, war
     _check(lib().turbofft_offline_ft_time(logN, _datatype(datatype), in_ptr, out_ptr, bs, warmup, reps, stream,
                                           C.byref(ms), C.byref(flagged)))
     return ms.value, flagged.value
+
+
+def membench_strided(write: bool, lane_bytes: int, run_bytes: int, log_stride: int, xcd_chunk: int, src_ptr: int, dst_ptr: int,
+                     nbytes: int, warmup: int = 2, reps: int = 10, stream: int = 0) -> float:
+    """ms per read-only or write-only pass over 64 KiB tiles made of `run_bytes` runs at a stride of 2^log_stride bytes."""
+    ms = C.c_float(0)
+    _check(lib().turbofft_membench_strided(int(bool(write)), lane_bytes, run_bytes, log_stride, xcd_chunk, src_ptr, dst_ptr, nbytes,
+                                           warmup, reps, stream, C.byref(ms)))
+    return ms.value
+
+
+def membench_fused(group: int, ring_slots: int, blocks_per_cu: int, src_ptr: int, scratch_ptr: int, scratch_bytes: int, dst_ptr: int,
+                   nbytes: int, limit_ms: int = 50, warmup: int = 1, reps: int = 5, stream: int = 0):
+    """Two-pass copy through a per-XCD ring as one persistent kernel: (ms per launch, stats dict)."""
+    ms = C.c_float(0)
+    st = (C.c_uint * 12)()
+    _check(lib().turbofft_membench_fused(group, ring_slots, blocks_per_cu, src_ptr, scratch_ptr, scratch_bytes, dst_ptr, nbytes, limit_ms,
+                                         warmup, reps, stream, C.byref(ms), st))
+    return ms.value, {"timed_out": st[0], "waits": st[1], "polls": st[2], "blocks": st[3], "blocks_per_xcd": list(st)[4:12]}
 
 
 def membench(mode: int, src_ptr: int, dst_ptr: int, nbytes: int, warmup: int = 2, reps: int = 10, stream: int = 0) -> float:

@@ -74,7 +74,223 @@ __global__ __launch_bounds__(256) void tfft_mb_write(V* __restrict__ out, int xc
     for (int e = 0; e < U; ++e) mb_st<AUX>(out + base, lane + (unsigned)(e * 256 * sizeof(V)), v);
 }
 
+// Strided tiles: 64 KiB made of rows of RUN bytes, row r of a tile at tile base + r << log_stride; tiles side by side
+// along a row first.  The access pattern of the column kernels (runs of BS elements at the stride of the digit) and
+// of the transposed store of the last launch.  Non-temporal, XCD-aware tile order.
+template <class V, int RUN, bool WRITE>
+__global__ __launch_bounds__(256) void tfft_mb_strided(const V* __restrict__ in, V* __restrict__ out, float* __restrict__ sink, int xcd_chunk, unsigned log_stride) {
+    constexpr unsigned W = sizeof(V), TILE = 65536, LPR = RUN / W, U = TILE / (256 * W);
+    const size_t t = mb_tile(xcd_chunk);
+    const unsigned tiles_per_row = (1u << log_stride) / RUN, rows = TILE / RUN;
+    const size_t base = (t / tiles_per_row) * rows * ((size_t)1 << log_stride) + (t % tiles_per_row) * RUN;       // bytes
+    const unsigned lane = (threadIdx.x % LPR) * W + ((threadIdx.x / LPR) << log_stride);
+    const unsigned step = (256 / LPR) << log_stride;
+    if (WRITE) {
+        V v;
+        v.x = (float)threadIdx.x;
+        v.y = 1.f;
+        if constexpr (sizeof(V) == 16) { v.z = (float)threadIdx.x; v.w = 1.f; }
+#pragma unroll
+        for (unsigned e = 0; e < U; ++e) mb_st<2>((V*)((char*)out + base), lane + e * step, v);
+    } else {
+        float acc = 0.f;
+#pragma unroll
+        for (unsigned e = 0; e < U; ++e) acc += mb_ld<2>((const V*)((const char*)in + base), lane + e * step).x;
+        if (acc == 123456.789f) sink[0] = acc;
+    }
+}
+
+// ---- two passes through a ring that stays in the XCD's L2 (the question a fused pass pair of a
+// two-launch plan would have to answer first) ----
+// Synthetic: in -> ring -> out as ONE persistent kernel.  The data is cut into "transforms" of 512 KiB;
+// each of the 8 XCDs (a block reads its XCD from the hardware register) owns every eighth transform and a
+// ring of R slots of G transforms that is reused for every group, so the intermediate is only ever written
+// to addresses that are still in that XCD's L2.  Items are handed out per XCD in ticket order
+//   P1(g0) | P1(g1) P2(g0) | P1(g2) P2(g1) | ...
+// (P1: 32 KiB of a transform in -> slot, 16 per transform; P2: 64 KiB slot -> out, 8 per transform).  A P2
+// item needs every P1 item of its group (as a row pass needs every column tile), a P1 item of group g
+// needs slot g % R drained by P2(g - R).  Every wait is for items with lower tickets, which running blocks
+// hold, so the order cannot deadlock whatever the grid; each wait is also bounded by a wall-clock limit after
+// which the block raises an error flag and every block leaves at its next ticket.
+constexpr long long kFusedTransform = 512 << 10;
+constexpr int kFusedP1 = 32 << 10, kFusedP2 = 64 << 10, kFusedMaxGroups = 2048;
+struct FusedQueue { unsigned next; unsigned pad0[31]; unsigned done1[kFusedMaxGroups]; unsigned done2[kFusedMaxGroups]; };
+struct FusedCtl { unsigned err, waits, spins, pad[29]; unsigned xcc_blocks[32]; FusedQueue q[8]; };
+
+__global__ void tfft_mb_fused_clear(FusedCtl* c) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < sizeof(FusedCtl) / 4) ((unsigned*)c)[i] = 0;
+}
+
+template <int U, int LAUX, int SAUX>
+__device__ __forceinline__ void fused_copy_item(const char* src, char* dst) {
+    u4 r[U];
+#pragma unroll
+    for (int e = 0; e < U; ++e) r[e] = __builtin_amdgcn_raw_buffer_load_b128(mb_rsrc(src), (threadIdx.x + e * 256) * 16u, 0, LAUX);
+#pragma unroll
+    for (int e = 0; e < U; ++e) __builtin_amdgcn_raw_buffer_store_b128(r[e], mb_rsrc(dst), (threadIdx.x + e * 256) * 16u, 0, SAUX);
+}
+
+// thread 0 waits until *p >= k; false after the time limit or when another block gave up
+__device__ __forceinline__ bool fused_wait(unsigned* p, unsigned k, FusedCtl* c, long long t_limit) {
+    unsigned spins = 0;
+    for (;;) {
+        if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= k) {
+            if (spins) { atomicAdd(&c->waits, 1u); atomicAdd(&c->spins, spins); }
+            return true;
+        }
+        if (__hip_atomic_load(&c->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+        if ((long long)wall_clock64() > t_limit) { atomicExch(&c->err, 1u); return false; }
+        __builtin_amdgcn_s_sleep(8);
+        ++spins;
+    }
+}
+
+__global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in, char* __restrict__ scratch, char* __restrict__ out, FusedCtl* c,
+                                                    int ntrans_per_xcd, int G, int R, int limit_ms) {
+    __shared__ unsigned s_t;
+    __shared__ int s_ok;
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;     // XCC_ID[3:0] of the hardware register
+    FusedQueue* q = &c->q[xcc];
+    const long long t_limit = (long long)wall_clock64() + (long long)limit_ms * 100000ll;   // 100 MHz counter
+    if (threadIdx.x == 0) atomicAdd(&c->xcc_blocks[xcc], 1u);
+    const int ngroups = ntrans_per_xcd / G;
+    const unsigned n1 = (unsigned)(kFusedTransform / kFusedP1 * G), n2 = (unsigned)(kFusedTransform / kFusedP2 * G);
+    const unsigned total = (unsigned)ngroups * (n1 + n2);
+    char* ring = scratch + (size_t)xcc * R * G * kFusedTransform;
+    for (;;) {
+        if (threadIdx.x == 0) {
+            unsigned t = atomicAdd(&q->next, 1u);
+            if (__hip_atomic_load(&c->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) t = 0xffffffffu;
+            s_t = t;
+        }
+        __syncthreads();
+        const unsigned t = (unsigned)__builtin_amdgcn_readfirstlane((int)s_t);
+        __syncthreads();
+        if (t >= total) break;
+        bool is1; unsigned g, i;
+        if (t < n1) { is1 = true; g = 0; i = t; }
+        else {
+            const unsigned u = t - n1, seg = u / (n1 + n2), r = u % (n1 + n2);
+            if (seg + 1 < (unsigned)ngroups) { if (r < n1) { is1 = true; g = seg + 1; i = r; } else { is1 = false; g = seg; i = r - n1; } }
+            else { is1 = false; g = (unsigned)ngroups - 1; i = r; }
+        }
+        char* slot = ring + (size_t)(g % R) * G * kFusedTransform;
+        if (is1) {
+            if (g >= (unsigned)R) {
+                if (threadIdx.x == 0) s_ok = fused_wait(&q->done2[g - R], n2, c, t_limit) ? 1 : 0;
+                __syncthreads();
+                const int ok = s_ok;
+                __syncthreads();
+                if (!ok) break;
+            }
+            const unsigned per = (unsigned)(kFusedTransform / kFusedP1), k = i / per, j = i % per;
+            const size_t T = (size_t)(g * G + k) * 8 + xcc;
+            fused_copy_item<kFusedP1 / 4096, 2, 0>(in + T * kFusedTransform + (size_t)j * kFusedP1, slot + (size_t)k * kFusedTransform + (size_t)j * kFusedP1);
+            __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): this wave's stores are acknowledged by the L2
+            __syncthreads();
+            if (threadIdx.x == 0) atomicAdd(&q->done1[g], 1u);
+        } else {
+            if (threadIdx.x == 0) s_ok = fused_wait(&q->done1[g], n1, c, t_limit) ? 1 : 0;
+            __syncthreads();
+            const int ok = s_ok;
+            __syncthreads();
+            if (!ok) break;
+            const unsigned per = (unsigned)(kFusedTransform / kFusedP2), k = i / per, j = i % per;
+            const size_t T = (size_t)(g * G + k) * 8 + xcc;
+            // agent-scope loads of the ring: never served from this CU's L1, which may hold the slot's previous contents
+            fused_copy_item<kFusedP2 / 4096, 16, 2>(slot + (size_t)k * kFusedTransform + (size_t)j * kFusedP2, out + T * kFusedTransform + (size_t)j * kFusedP2);
+            __builtin_amdgcn_s_waitcnt(0x0F70);       // the slot's loads have returned before it is handed back
+            __syncthreads();
+            if (threadIdx.x == 0) atomicAdd(&q->done2[g], 1u);
+        }
+    }
+}
+
+// `reps` timed launches between two events, after `warmup` untimed ones
+template <class F>
+int mb_time(F launch, int warmup, int reps, hipStream_t st, float* ms_per_pass, const char* what) {
+    for (int i = 0; i < warmup; ++i) launch();
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) { tfft_set_error("%s: hipEventCreate failed", what); return TURBOFFT_EHIP; }
+    if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); tfft_set_error("%s: hipEventCreate failed", what); return TURBOFFT_EHIP; }
+    hipError_t e = hipEventRecord(e0, st);
+    for (int i = 0; i < reps; ++i) launch();
+    if (e == hipSuccess) e = hipEventRecord(e1, st);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e == hipSuccess) e = hipGetLastError();
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess) { tfft_set_error("%s: %s", what, hipGetErrorString(e)); return TURBOFFT_EHIP; }
+    *ms_per_pass = ms / reps;
+    return TURBOFFT_OK;
+}
+
 }  // namespace
+
+extern "C" int turbofft_membench_strided(int write, int lane_bytes, int run_bytes, int log_stride, int xcd_chunk, const void* src_d,
+                                         void* dst_d, size_t bytes, int warmup, int reps, void* stream, float* ms_per_pass) {
+    if (!src_d || !dst_d || !ms_per_pass || reps < 1 || warmup < 0) { tfft_set_error("membench: bad argument"); return TURBOFFT_EINVAL; }
+    if ((lane_bytes != 8 && lane_bytes != 16) || (run_bytes != 128 && run_bytes != 256 && run_bytes != 512) || log_stride < 10 || log_stride > 22 ||
+        xcd_chunk < 0 || bytes == 0 || bytes % ((size_t)65536 / run_bytes << log_stride) || bytes / 65536 > 0x7fffffffull) {
+        tfft_set_error("membench: lanes of 8 or 16 bytes, runs of 128, 256 or 512 bytes, stride 2^10..2^22 bytes, bytes a multiple of (65536 / run) * stride");
+        return TURBOFFT_EINVAL;
+    }
+    const void* fns[2][2][3] = {
+        {{(const void*)tfft_mb_strided<v2, 128, false>, (const void*)tfft_mb_strided<v2, 256, false>, (const void*)tfft_mb_strided<v2, 512, false>},
+         {(const void*)tfft_mb_strided<v4, 128, false>, (const void*)tfft_mb_strided<v4, 256, false>, (const void*)tfft_mb_strided<v4, 512, false>}},
+        {{(const void*)tfft_mb_strided<v2, 128, true>, (const void*)tfft_mb_strided<v2, 256, true>, (const void*)tfft_mb_strided<v2, 512, true>},
+         {(const void*)tfft_mb_strided<v4, 128, true>, (const void*)tfft_mb_strided<v4, 256, true>, (const void*)tfft_mb_strided<v4, 512, true>}}};
+    const void* fn = fns[write ? 1 : 0][lane_bytes == 16][run_bytes == 128 ? 0 : (run_bytes == 256 ? 1 : 2)];
+    const unsigned grid = (unsigned)(bytes / 65536);
+    hipStream_t st = (hipStream_t)stream;
+    auto launch = [&]() {
+        const void* in_a = src_d; void* out_a = dst_d; float* sink = (float*)dst_d; int xca = xcd_chunk; unsigned ls = (unsigned)log_stride;
+        void* args[5] = {&in_a, &out_a, &sink, &xca, &ls};
+        (void)hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
+    };
+    return mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
+}
+
+extern "C" int turbofft_membench_fused(int group, int ring_slots, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+                                       void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
+                                       unsigned stats[12]) {
+    if (!src_d || !dst_d || !scratch_d || !ms_per_pass || !stats || reps < 1 || warmup < 0) { tfft_set_error("membench: bad argument"); return TURBOFFT_EINVAL; }
+    const long long ntrans = (long long)(bytes / kFusedTransform), per_xcd = ntrans / 8;
+    // (R >= 2: P1 of group g waits for P2 of group g - R, which has to come earlier in ticket order)
+    if (bytes == 0 || bytes % (8 * kFusedTransform) || group < 1 || ring_slots < 2 || ring_slots > 8 || per_xcd % group || per_xcd / group > kFusedMaxGroups ||
+        blocks_per_cu < 1 || blocks_per_cu > 8 || limit_ms < 1 || limit_ms > 1000 || (unsigned long long)8 * ring_slots * group * kFusedTransform > scratch_bytes) {
+        tfft_set_error("membench: fused copy needs bytes a multiple of 4 MiB, 2..8 ring slots of `group` 512 KiB transforms per XCD inside `scratch`, "
+                       "at most %d groups per XCD, 1..8 blocks per CU and a time limit of 1..1000 ms", kFusedMaxGroups);
+        return TURBOFFT_EINVAL;
+    }
+    int dev = 0, cus = 0, occ = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, tfft_mb_fused, 256, 0) != hipSuccess || occ < 1) {
+        (void)hipGetLastError();
+        tfft_set_error("membench: cannot size the persistent grid");
+        return TURBOFFT_EHIP;
+    }
+    if (blocks_per_cu > occ) blocks_per_cu = occ;
+    FusedCtl* ctl = nullptr;
+    if (hipMalloc((void**)&ctl, sizeof(FusedCtl)) != hipSuccess) { (void)hipGetLastError(); tfft_set_error("membench: hipMalloc failed"); return TURBOFFT_ENOMEM; }
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)(cus * blocks_per_cu);
+    auto launch = [&]() {
+        hipLaunchKernelGGL(tfft_mb_fused_clear, dim3((unsigned)((sizeof(FusedCtl) / 4 + 255) / 256)), dim3(256), 0, st, ctl);
+        hipLaunchKernelGGL(tfft_mb_fused, dim3(grid), dim3(256), 0, st, (const char*)src_d, (char*)scratch_d, (char*)dst_d, ctl, (int)per_xcd, group, ring_slots, limit_ms);
+    };
+    int rc = mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
+    unsigned head[64];
+    if (rc == TURBOFFT_OK && hipMemcpy(head, ctl, sizeof head, hipMemcpyDeviceToHost) != hipSuccess) { (void)hipGetLastError(); tfft_set_error("membench: reading the control block failed"); rc = TURBOFFT_EHIP; }
+    (void)hipFree(ctl);
+    if (rc) return rc;
+    stats[0] = head[0]; stats[1] = head[1]; stats[2] = head[2]; stats[3] = grid;      // error flag, waits, polls, blocks
+    for (int x = 0; x < 8; ++x) stats[4 + x] = head[32 + x];                          // blocks that ran on each XCD
+    return TURBOFFT_OK;
+}
 
 extern "C" int turbofft_membench(int mode, const void* src_d, void* dst_d, size_t bytes, int warmup, int reps,
                                  void* stream, float* ms_per_pass) {
@@ -103,20 +319,5 @@ extern "C" int turbofft_membench(int mode, const void* src_d, void* dst_d, size_
         if (kind == 3) { void* args[2] = {&out_a, &xca}; (void)hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds, st); }
         else { void* args[3] = {&in_a, &out_a, &xca}; (void)hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds, st); }
     };
-    for (int i = 0; i < warmup; ++i) launch();
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess) { tfft_set_error("membench: hipEventCreate failed"); return TURBOFFT_EHIP; }
-    if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); tfft_set_error("membench: hipEventCreate failed"); return TURBOFFT_EHIP; }
-    hipError_t e = hipEventRecord(e0, st);
-    for (int i = 0; i < reps; ++i) launch();
-    if (e == hipSuccess) e = hipEventRecord(e1, st);
-    if (e == hipSuccess) e = hipEventSynchronize(e1);
-    float ms = 0;
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e == hipSuccess) e = hipGetLastError();
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    if (e != hipSuccess) { tfft_set_error("membench: %s", hipGetErrorString(e)); return TURBOFFT_EHIP; }
-    *ms_per_pass = ms / reps;
-    return TURBOFFT_OK;
+    return mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
 }
