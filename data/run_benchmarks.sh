@@ -28,4 +28,7 @@ for dt in 0 1; do
     for t in 1 2 4 8 16 32; do
         run "$out/ft/ft_scheme_threadblock_bs=${t}_${gpu}_$p.csv" "turboFFT," --if_bench 1 --thread_bs $t --datatype $dt --if_ft 1 --if_err 1
     done
+    # thread-level verification (the scheme of the reference's data_ft/ft_scheme_thread_bs=1_*): clean, and with the injection cadence
+    run "$out/benchmark_TurboFFT_thread_level_${gpu}_$p.csv" "turboFFT," --if_bench 2 --thread_bs 1 --datatype $dt --if_ft 1 --if_err 0 --ft_scheme 1
+    run "$out/ft/ft_scheme_thread_bs=1_${gpu}_$p.csv"        "turboFFT," --if_bench 1 --thread_bs 1 --datatype $dt --if_ft 1 --if_err 1 --ft_scheme 1
 done
