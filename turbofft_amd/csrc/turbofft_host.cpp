@@ -23,6 +23,7 @@
 
 extern "C" const char* tfft_builtin_param_csv(int datatype);   // generated: the gfx950 CSV text
 extern "C" const char* tfft_builtin_param_ft_csv(int datatype);   // generated: rows replaced in FT plans
+extern "C" const char* tfft_builtin_param_tt_csv(int datatype);   // generated: rows replaced in plans with thread-level verification
 extern "C" const char* tfft_builtin_param_small_csv(int datatype);   // generated: rows for batches too small to fill the device
 
 namespace {
@@ -407,6 +408,14 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             std::istringstream fin(tfft_builtin_param_ft_csv(p->datatype));
             std::vector<Row> repl;
             if (!parse_csv(fin, repl)) return fail(TURBOFFT_ENOPLAN, "built-in fault-tolerant plan table is malformed");
+            for (const Row& r : repl)
+                if (r.logN() >= 0 && r.logN() < (int)rows.size()) rows[r.logN()] = r;
+        } else if (p->if_ft) {
+            // thread-level verification runs the plain rows, except where its two sums beside the data cost a
+            // wavefront per SIMD and another shape measured faster
+            std::istringstream fin(tfft_builtin_param_tt_csv(p->datatype));
+            std::vector<Row> repl;
+            if (!parse_csv(fin, repl)) return fail(TURBOFFT_ENOPLAN, "built-in thread-level plan table is malformed");
             for (const Row& r : repl)
                 if (r.logN() >= 0 && r.logN() < (int)rows.size()) rows[r.logN()] = r;
         }
