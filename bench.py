@@ -245,6 +245,56 @@ def sweep_rows(torch, turbofft_amd, lo=7, hi=24, steps=10, ft_rounds=2, ft_block
     return rows
 
 
+def fused_pair_rows(torch, turbofft_amd, steps=10, rounds=4, log=None):
+    """The sizes whose two launches also exist as one kernel (plans created with TURBOFFT_FUSED=1 hold it): that kernel
+    against the plan's two launches at logBS+logN=28, in alternating blocks of `steps` event-timed executions."""
+    rows = []
+    stream = torch.cuda.current_stream().cuda_stream
+    before = os.environ.get("TURBOFFT_FUSED")
+    os.environ["TURBOFFT_FUSED"] = "1"
+    try:
+        for dt, logN in ((0, 16), (1, 15), (1, 16)):
+            plan = turbofft_amd.TurboFFT(logN, dt)
+            if plan.fused_info() is None:
+                plan.close()
+                continue
+            bs = 1 << (28 - logN)
+            x = make_input(torch, bs, 1 << logN, dt)
+            out = torch.empty(2 << 28, dtype=torch.complex64 if dt == 0 else torch.complex128, device="cuda")
+            ms = {True: [], False: []}
+            names = {}
+            for rnd in range(rounds):
+                for fused in (True, False):
+                    plan.set_fused(fused)
+                    names[fused] = plan.kernel_names_for_batch(bs)
+                    for _ in range(3):
+                        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(steps):
+                        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    ms[fused].append(e0.elapsed_time(e1) / steps)
+            f, t = stats(ms[True])["median"], stats(ms[False])["median"]
+            row = {"logN": logN, "dtype": "f32" if dt == 0 else "f64", "bs": bs, "fused_kernel": names[True][0], "ms_fused": f, "ms_two_launches": t,
+                   "two_launches_over_fused": t / f, "gbs_fused": plan.gbs(bs, f), "team": plan.fused_info() or None}
+            plan.set_fused(True)
+            row["team"] = plan.fused_info()
+            plan.close()
+            rows.append(row)
+            if log:
+                log(row)
+            del x, out
+            torch.cuda.empty_cache()
+    finally:
+        if before is None:
+            del os.environ["TURBOFFT_FUSED"]
+        else:
+            os.environ["TURBOFFT_FUSED"] = before
+    return rows
+
+
 def cpu_baseline(logN, datatype, target_s=10.0):
     """Reference CPU path: pocketfft via scipy.fft on all host cores the box
     gives one GPU (16), on a bounded sample of the workload."""
@@ -326,6 +376,9 @@ def main():
     ap.add_argument("--membench_fused", type=str, default=None, metavar="G:R:B",
                     help="--membench: only the two-pass copy through a per-XCD ring of R slots of G 512 KiB pieces with B blocks per CU "
                          "(for counter runs of one configuration)")
+    ap.add_argument("--membench_team", type=str, default=None, metavar="T:P:B",
+                    help="--membench: only the two-pass copy with teams of T blocks that share a slot of P KiB, B blocks per CU")
+    ap.add_argument("--fused_pairs", action="store_true", help="only the fused-pair comparison (one JSON line)")
     ap.add_argument("--calib_copy", type=int, default=0,
                     help="also run this many plain device copies of the input (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -348,12 +401,15 @@ def main():
             turbofft_amd.membench(0, src.data_ptr(), dst.data_ptr(), nbytes, 0, 10, st)      # clock the device up
         res = {}
         only_fused = [tuple(int(t) for t in a.membench_fused.split(":"))] if a.membench_fused else None
+        only_team = [tuple(int(t) for t in a.membench_team.split(":"))] if a.membench_team else None
+        if only_team:
+            only_fused = []
         # every kernel plain, then with what the FFT kernels use: non-temporal accesses (+4), XCD-aware
         # tile order (+8) and a bound on the blocks resident per CU (+16*k; the exchange buffer of an
         # FFT kernel bounds it to 2-4)
         flavours = (("", 0), ("_nt", 4), ("_nt_xcd", 12), ("_nt_xcd_2percu", 12 + 32), ("_nt_xcd_3percu", 12 + 48), ("_nt_xcd_4percu", 12 + 64), ("_nt_xcd_6percu", 12 + 96))
         for kind, name, moved in ((0, "copy_8B_lanes", 2), (1, "copy_16B_lanes", 2), (2, "read_only", 1), (3, "write_only", 1)):
-            if only_fused:
+            if only_fused is not None:
                 break
             for sfx, bits in flavours:
                 ms = sorted(turbofft_amd.membench(kind + bits, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))
@@ -361,7 +417,7 @@ def main():
                 print(f"{name + sfx:32s} {ms[2]:.4f} ms  {moved * nbytes / ms[2] / 1e6:7.0f} GB/s", file=sys.stderr, flush=True)
         # the access patterns of the column kernels and of the transposed store: runs of 128-512 bytes at a large stride
         strided = {}
-        for ls in (() if only_fused else (12, 14, 16, 19)):
+        for ls in (() if only_fused is not None else (12, 14, 16, 19)):
             for run in (128, 256, 512):
                 for lane in (8, 16):
                     for write in (0, 1):
@@ -379,7 +435,7 @@ def main():
         fused = {}
         two = sorted(turbofft_amd.membench(12, src.data_ptr(), dst.data_ptr(), nbytes, 3, 20, st) for _ in range(5))[2] * 2
         fused["two_whole_passes_ms"] = two
-        for G, R, bpc in (only_fused or ((1, 3, 2), (2, 3, 2), (4, 2, 2), (4, 3, 2), (8, 3, 2), (8, 3, 3))):
+        for G, R, bpc in (only_fused if only_fused is not None else ((1, 3, 2), (2, 3, 2), (4, 2, 2), (4, 3, 2), (8, 3, 2), (8, 3, 3))):
             dst.zero_()
             ms, stt = turbofft_amd.membench_fused(G, R, bpc, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, 50, 1, 5, st)
             ok = bool(torch.equal(src, dst))
@@ -387,7 +443,22 @@ def main():
             print(f"fused copy: {G} x 512 KiB per group, {R} slots ({G * R * 512} KiB ring per XCD), {bpc} blocks per CU: {ms:.3f} ms "
                   f"(two whole passes {two:.3f} ms), right {ok}, {stt}", file=sys.stderr, flush=True)
         res["fused_two_pass_copy"] = fused
+        # the same two passes with teams of blocks that share ONE slot each (the form the fused FFT kernels use)
+        team = {}
+        scratch = torch.empty((8 * 64 * 1024 * 1024) // 4, device="cuda", dtype=torch.float32)
+        for T, P, bpc in (only_team or ((() if a.membench_fused else ((4, 256, 1), (4, 256, 2), (8, 512, 1), (8, 512, 2), (16, 512, 2), (8, 1024, 1), (16, 1024, 1), (16, 1024, 2))))):
+            dst.zero_()
+            ms, stt = turbofft_amd.membench_team(T, bpc, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, 50, 1, 5, st, piece_kib=P)
+            ok = bool(torch.equal(src, dst))
+            slots = (stt["blocks"] // 8) // T
+            team[f"team{T}_piece{P}KiB_blocks{bpc}"] = {"ms": ms, "slots_KiB_per_xcd": slots * P, "copied_right": ok, **stt}
+            print(f"team copy: teams of {T}, pieces of {P} KiB, {bpc} blocks per CU ({slots * P} KiB of slots per XCD): {ms:.3f} ms "
+                  f"(two whole passes {two:.3f} ms), right {ok}, us per round {stt['us_per_round']}", file=sys.stderr, flush=True)
+        res["team_two_pass_copy"] = team
         print(json.dumps({"membench": res, "bytes": nbytes, "tile_bytes": 65536, "threads": 256}), flush=True)
+        return 0
+    if a.fused_pairs:
+        print(json.dumps({"fused_pairs": fused_pair_rows(torch, turbofft_amd, max(10, a.sweep_steps))}), flush=True)
         return 0
     if a.sweep:
         lines = []
@@ -491,9 +562,11 @@ def main():
     del x, out
     torch.cuda.empty_cache()
     sweep = None
+    fused_pairs = None
     if not a.no_sweep and not (a.if_ft or a.if_err):
         t_sw = time.perf_counter()
         sweep = sweep_rows(torch, turbofft_amd, a.sweep_lo, a.sweep_hi, max(10, a.sweep_steps))
+        fused_pairs = fused_pair_rows(torch, turbofft_amd, max(10, a.sweep_steps))
         sweep_s = time.perf_counter() - t_sw
     tname = "fp32" if dt == 0 else "fp64"
     launches = r["launches"]
@@ -520,6 +593,7 @@ def main():
     }
     if sweep is not None:
         line["sweep"] = sweep
+        line["fused_pairs"] = fused_pairs         # opt-in kernels (TURBOFFT_FUSED=1): both launches of a two-launch plan in one
         line["sweep_s"] = sweep_s
     if sync_ms is not None:
         line["ms_per_step_sync_each_launch"] = sync_ms          # main.cu:53-62 protocol, reported only

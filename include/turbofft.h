@@ -355,16 +355,49 @@ int turbofft_membench_strided(int write, int lane_bytes, int run_bytes, int log_
 
 /* Two passes through a ring that is meant to stay in the XCD's L2: a copy src -> ring -> dst as ONE persistent
  * kernel (`blocks_per_cu` blocks per CU), the data cut into 512 KiB pieces that the 8 XCDs own in turn, each XCD
- * with `ring_slots` (2..8) slots of `group` pieces inside `scratch_d` (8 * ring_slots * group * 512 KiB), reused for
+ * with `ring_slots` (lag+1..16) slots of `group` pieces inside `scratch_d` (8 * ring_slots * group * 512 KiB), reused for
  * every group; the second pass of a group starts when its first pass is complete, as the row pass of a two-launch
- * plan needs every column tile of its transform.  Measures whether a fused pass pair could keep its intermediate
+ * plan needs every column tile of its transform, and is handed out `lag` groups behind the first pass, so that with a
+ * large enough lag no block finds a group's first pass still running.  Measures whether a fused pass pair could keep its intermediate
  * on chip (rocprofv3's FETCH_SIZE / WRITE_SIZE of the kernel tell where the ring's traffic went).  Every wait inside
  * the kernel is for work that running blocks hold and is bounded by `limit_ms` per launch: on a time-out the kernel
  * drains and stats[0] is 1.  stats: [0] time-out flag, [1] waits that had to poll, [2] polls, [3] blocks launched,
  * [4..11] blocks that ran on each XCD.  dst equals src afterwards.  `bytes` is a multiple of 4 MiB. */
-int turbofft_membench_fused(int group, int ring_slots, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+int turbofft_membench_fused(int group, int ring_slots, int lag, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
                             void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
                             unsigned stats[12]);
+
+/* The same copy with teams instead of tickets: `team_blocks` (4, 8, 16, 32) blocks of one XCD share one piece of
+ * `piece_kib` KiB (128, 256, 512, 1024; 4..128 KiB per member) at a time and one slot of `scratch_d` (blocks per XCD /
+ * team_blocks slots per XCD), meeting at a team barrier between the pass that fills the slot and the pass that drains
+ * it (each member drains a strip of every member's part) and again before the slot is overwritten.  The whole grid
+ * (`blocks_per_cu`, at most what fits) has to be resident at once; waits are bounded by `limit_ms` as in
+ * turbofft_membench_fused.  stats: [0] time-out flag, [1] waits that had to poll, [2] polls, [3] blocks launched, [4..9] mean
+ * time per round, in units of 10 ns, that a block spends waiting for the piece's loads, waiting for the slot, on the slot's
+ * stores, in the team barrier, on the slot's loads, on the rest, [10] rounds per block.  `bytes` is a multiple of 8 pieces.  `policy` (teams of 8
+ * with pieces of 512 KiB only, else 0) picks the cache policy of the accesses to memory: loads of src in bits 0-1,
+ * stores to dst in bits 2-3, each 0 non-temporal, 1 that with sc0, 2 with sc1, 3 with both. */
+int turbofft_membench_team(int team_blocks, int piece_kib, int policy, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+                           void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
+                           unsigned stats[12]);
+
+/* Fused pairs.  For some sizes a plain built-in two-launch plan also holds ONE kernel that runs both launches
+ * (param/gfx950/param_<T>_pair.csv): teams of blocks on one XCD take pieces of a few whole transforms from a queue,
+ * run the column launch of a piece into a slot that the XCD's L2 holds, meet, and run the row launch out of the slot,
+ * so the plan's intermediate never travels to memory.  It runs for batches that give every team a piece; `out` may
+ * then hold N*bs elements only.  Every block of its grid has to be resident at once: it is sized for a GPU it has to
+ * itself, shares the CUs with other kernels correctly as long as those finish on their own, and bounds every wait
+ * (TURBOFFT_FUSED_LIMIT_MS, default 2000): should the limit ever be reached the output of that execution is
+ * incomplete, the next turbofft_exec on that stream returns TURBOFFT_EHIP saying so, and the plan goes back to its
+ * two launches.  Every stream that runs the fused kernel owns a set of slots (8 sets per plan; later streams, and
+ * streams that first show up while being captured, run the two launches).
+ * turbofft_plan_set_fused switches it off or on for a plan; TURBOFFT_FUSED=0 in the environment leaves it out of
+ * new plans.  turbofft_plan_fused_info returns 1 when the plan holds an enabled fused kernel, 0 when not, and fills
+ * in (where non-null) the blocks per team, transforms per piece, teams per XCD and blocks of its grid.
+ * No counterpart in the reference, whose multi-launch plans always store and reload the intermediate
+ * (main.cu:16-30). */
+int turbofft_plan_set_fused(turbofft_plan_t* plan, int enable);
+int turbofft_plan_fused_info(const turbofft_plan_t* plan, int* team_blocks, int* transforms_per_piece, int* teams_per_xcd, int* grid_blocks);
 
 /* The `turbofft` command line (main.cu:137-169 + CommandLineParser.h): same
  * flags and output lines.  Returns the process exit code. */

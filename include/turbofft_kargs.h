@@ -79,6 +79,38 @@ typedef struct tfft_kargs {
     tfft_ft_args ft;
 } tfft_kargs;
 
+/* Extra argument of a fused pair: one kernel that runs both launches of a two-launch plan.  A team of
+ * `team` blocks of one XCD takes pieces of `piece_elems` elements (whole transforms) from a queue, runs
+ * the column launch of a piece into the team's slot (slot k of `slots`, piece_elems elements each, meant
+ * to stay in that XCD's L2), meets, and runs the row launch out of the slot.  `ctl` is the control block
+ * (32-bit words, 128-byte lines so that no two counters share one; all zero between launches: the last
+ * block to leave clears it):
+ *   word 0                    set when a wait ran out of time (the output is then incomplete; err_host keeps the fact)
+ *   word 32                   the next piece of the queue
+ *   word 64                   blocks that have left
+ *   word 96 + 32 * x          blocks that have arrived on XCD x (x < 8)
+ *   word 352 + 128 * slot     + 0: members that finished the column launch, + 32: members that finished
+ *                             reading the slot, + 64 and + 96 (two words each): the piece of even and of odd
+ *                             rounds, (round + 1) << 32 | piece + 1 as named by the team's first member, piece + 1 = 0
+ *                             when the queue is empty
+ * A block that arrives when its XCD's `teams_per_xcd` teams are full has nothing to do. */
+typedef struct tfft_fuse_args {
+    void* slots;
+    unsigned* ctl;
+    unsigned* err_host;           /* host-visible word set together with word 0 of ctl (may be null) */
+    long long piece_elems;
+    long long npieces;
+    int tiles_a, tiles_b;         /* tiles of the column launch and of the row launch per piece        */
+    int team;                     /* blocks per team                                                  */
+    int teams_per_xcd;
+    int limit_ms;                 /* longest time a block waits for other blocks                      */
+    unsigned long long* prof;     /* diagnostic builds of the kernels only (else null): 8 words per block, ticks of the
+                                     100 MHz counter spent in [0] the column launch, [1] the meeting, [2] the row launch,
+                                     [3] the wait for the slot to be free, [4] rounds                                 */
+} tfft_fuse_args;
+
+#define TFFT_FUSE_CTL_WORDS(slots) (352 + 128 * (slots))
+
 #ifdef __cplusplus
 }
 #endif

@@ -147,3 +147,59 @@ def split_tables(logL, dtype):
     hi = np.exp(-2j * np.pi * (np.arange(1 << (logL - lo_bits)) << lo_bits) / L)
     lo = np.exp(-2j * np.pi * np.arange(1 << lo_bits) / L)
     return lo_bits, hi.astype(ctype_of(dtype)), lo.astype(ctype_of(dtype))
+
+
+class FuseArgs(C.Structure):
+    _fields_ = [("slots", C.c_void_p), ("ctl", C.c_void_p), ("err_host", C.c_void_p), ("piece_elems", C.c_longlong),
+                ("npieces", C.c_longlong), ("tiles_a", C.c_int), ("tiles_b", C.c_int), ("team", C.c_int),
+                ("teams_per_xcd", C.c_int), ("limit_ms", C.c_int)]
+
+
+def run_pair_sim(fs, x_in: np.ndarray, bs: int, team: int, per_piece: int):
+    """The fused pair of a two-launch plan for `bs` transforms of 2^(logN1 + logN2) points, one team of
+    `team` members working through pieces of `per_piece` transforms (the last piece may be ragged)."""
+    from turbofft_amd.codegen.fft_codegen import generate_fused_source
+    src = generate_fused_source(fs, True).replace(
+        '#include "../tfft_device.h"', f'#include "{ROOT}/turbofft_amd/csrc/tfft_device.h"')
+    src += "\ntfft_sim_bounds_t tfft_sim_bounds; long long tfft_sim_errors = 0;\n"
+    src += 'extern "C" long long tfft_sim_error_count() { return tfft_sim_errors; }\n'
+    h = hashlib.sha1(src.encode()).hexdigest()[:16]
+    os.makedirs(_CACHE, exist_ok=True)
+    so = os.path.join(_CACHE, f"{fs.name}_{h}.so")
+    if not os.path.exists(so):
+        tmp = f"{so[:-3]}.{os.getpid()}"
+        with open(tmp + ".cpp", "w") as f:
+            f.write(src)
+        subprocess.check_call(["g++", "-O1", "-shared", "-fPIC", "-o", tmp + ".so", tmp + ".cpp"])
+        os.replace(tmp + ".so", so)
+        os.remove(tmp + ".cpp")
+    lib = C.CDLL(so)
+    dtype = fs.T2
+    ct = ctype_of(dtype)
+    l1, l2 = fs.a.logNi, fs.b.logNi
+    N = 1 << (l1 + l2)
+    x_in = np.ascontiguousarray(x_in, dtype=ct).ravel()
+    assert x_in.size == bs * N
+    out = np.full(bs * N, np.nan + 1j * np.nan, dtype=ct)
+    slot = np.full(per_piece * N, np.nan + 1j * np.nan, dtype=ct)
+    tw = twiddle_table(max(1 << l1, 1 << l2), dtype)
+    lo_bits, hi, lo = split_tables(l1 + l2, dtype)
+    a0, a1 = KArgs(), KArgs()
+    a0.ntiles, a0.thread_bs, a0.tb_gap, a0.log_ncols, a0.tw_lo_bits = bs * ((1 << l2) // fs.a.BS), 1, 1, l2, lo_bits
+    a0.tw_hi, a0.tw_lo = hi.ctypes.data, lo.ctypes.data
+    a1.ntiles, a1.thread_bs, a1.tb_gap = bs * ((1 << l1) // fs.b.BS), 1, 1
+    a1.logQ, a1.logC, a1.logN = 0, l1, l1 + l2
+    f = FuseArgs()
+    f.piece_elems, f.npieces = per_piece * N, (bs + per_piece - 1) // per_piece
+    f.tiles_a, f.tiles_b = per_piece * ((1 << l2) // fs.a.BS), per_piece * ((1 << l1) // fs.b.BS)
+    f.team, f.teams_per_xcd, f.limit_ms = team, 1, 1
+    lim = np.zeros(6, dtype=np.int64)
+    lim[0], lim[1], lim[2], lim[3], lim[4] = x_in.size, out.size, tw.size, hi.size, lo.size
+    fn = getattr(lib, fs.name + "_sim")
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(KArgs), C.POINTER(KArgs), C.POINTER(FuseArgs), C.c_void_p, C.c_void_p]
+    fn.restype = None
+    fn(x_in.ctypes.data, out.ctypes.data, tw.ctypes.data, C.byref(a0), C.byref(a1), C.byref(f), slot.ctypes.data, lim.ctypes.data)
+    lib.tfft_sim_error_count.restype = C.c_longlong
+    errs = lib.tfft_sim_error_count()
+    assert errs == 0, f"{errs} out-of-bounds accesses in {fs.name}"
+    return out.reshape(bs, N)

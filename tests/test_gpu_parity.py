@@ -848,3 +848,111 @@ def test_streaming_yardsticks_run():
         turbofft_amd.membench_fused(4, 3, 2, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes)
     with pytest.raises(turbofft_amd.TurboFFTError):           # one slot: a first pass would wait for a later ticket
         turbofft_amd.membench_fused(1, 1, 2, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes)
+    # the same copy with teams of blocks that share one slot: right for every team size and piece, never out of time
+    scratch = torch.empty((64 << 20) // 4, device="cuda", dtype=torch.float32)
+    for T, piece, bpc in ((8, 512, 1), (4, 256, 2), (16, 1024, 1), (32, 128, 4)):
+        dst.zero_()
+        ms, stats = turbofft_amd.membench_team(T, bpc, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, 200, 1, 2, st, piece_kib=piece)
+        assert ms > 0 and stats["timed_out"] == 0 and stats["rounds_per_block"] > 0
+        assert torch.equal(src, dst)
+    with pytest.raises(turbofft_amd.TurboFFTError):           # a member's share of the piece would not fit its registers
+        turbofft_amd.membench_team(4, 1, src.data_ptr(), scratch.data_ptr(), scratch.numel() * 4, dst.data_ptr(), nbytes, piece_kib=1024)
+
+
+FUSED = [("float2", 16), ("double2", 15), ("double2", 16)]
+
+
+@pytest.mark.parametrize("dt,logN", FUSED)
+def test_fused_pair_matches_the_dft_and_the_two_launches(dt, logN, monkeypatch):
+    # a plan created with TURBOFFT_FUSED=1 holds ONE kernel for both launches of these sizes (teams of blocks pass the
+    # intermediate through a slot in their XCD's L2); it runs for batches that give every team a piece
+    torch = _torch()
+    monkeypatch.setenv("TURBOFFT_FUSED", "1")
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    info = plan.fused_info()
+    assert info is not None and info["grid_blocks"] == 8 * info["teams_per_xcd"] * info["team_blocks"]
+    teams = 8 * info["teams_per_xcd"] * info["transforms_per_piece"]
+    assert plan.launches == 2 and len(plan.kernel_names_for_batch(teams)) == 1 and "_pair_" in plan.kernel_names_for_batch(teams)[0]
+    assert plan.kernel_names_for_batch(teams - 1) == plan.kernel_names()           # too few pieces: the two launches
+    for bs, seed in ((teams, 1), (3 * teams + 5, 2), (teams - 1, 3)):
+        x = make(bs, 1 << logN, dt, seed)
+        y = gpu_fft(plan, x)
+        assert O.rel_l2(y, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    # against the plan's two launches on the same input: the same transform to rounding, on an output of N*bs elements only
+    bs = 2 * teams + 1
+    x = torch.from_numpy(make(bs, 1 << logN, dt, 9)).cuda()
+    out = torch.zeros(2 * bs << logN, dtype=x.dtype, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    for rep in range(3):                                                        # the control block is left clean for the next launch
+        out.zero_()
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, st)
+    torch.cuda.synchronize()
+    assert not bool(out[bs << logN:].any())                                     # no intermediate in the caller's buffer
+    out = out[: bs << logN]
+    plan.set_fused(False)
+    assert plan.fused_info() is None and len(plan.kernel_names_for_batch(bs)) == 2
+    two = plan.fft(x)
+    torch.cuda.synchronize()
+    assert O.rel_l2(out.view(bs, -1).cpu().numpy(), two.cpu().numpy()) <= O.tolerance(dt, logN)
+    plan.set_fused(True)
+    plan.close()
+    # without the variable a plan holds no fused kernel and says so
+    monkeypatch.delenv("TURBOFFT_FUSED")
+    plain = turbofft_amd.TurboFFT(logN, dt)
+    assert plain.fused_info() is None
+    with pytest.raises(turbofft_amd.TurboFFTError):
+        plain.set_fused(True)
+    plain.close()
+
+
+def test_fused_pair_on_several_streams_and_in_a_graph(monkeypatch):
+    # every stream that runs the fused kernel owns its slots and control block (eight sets per plan, later streams
+    # run the two launches); a stream that first shows up while it is being captured gets none and records the two launches
+    torch = _torch()
+    monkeypatch.setenv("TURBOFFT_FUSED", "1")
+    dt, logN = "float2", 16
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    info = plan.fused_info()
+    bs = 8 * info["teams_per_xcd"] + 3
+    xs = [torch.from_numpy(make(bs, 1 << logN, dt, 300 + i)).cuda() for i in range(10)]
+    want = [O.fft_ref(x.cpu().numpy()) for x in xs]
+    outs = [torch.zeros(plan.out_elems(bs), dtype=x.dtype, device="cuda") for x in xs]
+    streams = [torch.cuda.Stream() for _ in xs]
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for x, o, s in zip(xs, outs, streams):
+            plan.exec(x.data_ptr(), o.data_ptr(), bs, s.cuda_stream)
+    torch.cuda.synchronize()
+    for o, w in zip(outs, want):
+        assert O.rel_l2(o[: bs << logN].view(bs, -1).cpu().numpy(), w) <= O.tolerance(dt, logN)
+    plan.close()
+    # capture on a stream the plan has not seen (its first set belongs to the default stream by then)
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    x = xs[0]
+    eager = plan.fft(x).clone()
+    out = torch.zeros(plan.out_elems(bs), dtype=x.dtype, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream().cuda_stream)
+    for rep in range(2):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert O.rel_l2(out[: bs << logN].view(bs, -1).cpu().numpy(), want[0]) <= O.tolerance(dt, logN)
+    # and on a stream that owns a set: the fused kernel itself is captured (it clears its own control block)
+    with torch.cuda.stream(stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, stream.cuda_stream)
+    stream.synchronize()
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2, stream=stream):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out[: bs << logN].view(bs, -1), eager)
+    plan.close()

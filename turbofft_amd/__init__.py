@@ -74,6 +74,8 @@ def lib() -> C.CDLL:
     L.turbofft_plan_small_batch_max.argtypes = [vp]
     L.turbofft_plan_small_batch_max.restype = ll
     L.turbofft_plan_set_small_batch.argtypes = [vp, i]
+    L.turbofft_plan_set_fused.argtypes = [vp, i]
+    L.turbofft_plan_fused_info.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
     L.turbofft_plan_kernel_name.argtypes = [vp, i]
     L.turbofft_plan_kernel_name.restype = C.c_char_p
     L.turbofft_plan_launches_for_batch.argtypes = [vp, ll]
@@ -97,7 +99,8 @@ def lib() -> C.CDLL:
     L.turbofft_vendor_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_membench.argtypes = [i, vp, vp, C.c_size_t, i, i, vp, C.POINTER(C.c_float)]
     L.turbofft_membench_strided.argtypes = [i, i, i, i, i, vp, vp, C.c_size_t, i, i, vp, C.POINTER(C.c_float)]
-    L.turbofft_membench_fused.argtypes = [i, i, i, vp, vp, C.c_size_t, vp, C.c_size_t, i, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_uint)]
+    L.turbofft_membench_fused.argtypes = [i, i, i, i, vp, vp, C.c_size_t, vp, C.c_size_t, i, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_uint)]
+    L.turbofft_membench_team.argtypes = [i, i, i, i, vp, vp, C.c_size_t, vp, C.c_size_t, i, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_uint)]
     L.turbofft_offline_checksums.argtypes = [i, i, vp, vp, ll, vp, vp, vp]
     L.turbofft_offline_ft_time.argtypes = [i, i, vp, vp, ll, i, i, vp, C.POINTER(C.c_float), C.POINTER(C.c_ulonglong)]
     _lib = L
@@ -202,13 +205,26 @@ def membench_strided(write: bool, lane_bytes: int, run_bytes: int, log_stride: i
 
 
 def membench_fused(group: int, ring_slots: int, blocks_per_cu: int, src_ptr: int, scratch_ptr: int, scratch_bytes: int, dst_ptr: int,
-                   nbytes: int, limit_ms: int = 50, warmup: int = 1, reps: int = 5, stream: int = 0):
+                   nbytes: int, limit_ms: int = 50, warmup: int = 1, reps: int = 5, stream: int = 0, lag: int = 1):
     """Two-pass copy through a per-XCD ring as one persistent kernel: (ms per launch, stats dict)."""
     ms = C.c_float(0)
     st = (C.c_uint * 12)()
-    _check(lib().turbofft_membench_fused(group, ring_slots, blocks_per_cu, src_ptr, scratch_ptr, scratch_bytes, dst_ptr, nbytes, limit_ms,
+    _check(lib().turbofft_membench_fused(group, ring_slots, lag, blocks_per_cu, src_ptr, scratch_ptr, scratch_bytes, dst_ptr, nbytes, limit_ms,
                                          warmup, reps, stream, C.byref(ms), st))
     return ms.value, {"timed_out": st[0], "waits": st[1], "polls": st[2], "blocks": st[3], "blocks_per_xcd": list(st)[4:12]}
+
+
+def membench_team(team_blocks: int, blocks_per_cu: int, src_ptr: int, scratch_ptr: int, scratch_bytes: int, dst_ptr: int, nbytes: int,
+                  limit_ms: int = 50, warmup: int = 1, reps: int = 5, stream: int = 0, piece_kib: int = 512, policy: int = 0):
+    """Two-pass copy through one L2-resident slot per team of blocks: (ms per launch, stats dict).  stats["us_per_round"]
+    is the mean time a block spends per round in: waiting for the piece's loads, waiting for the slot, the slot's stores,
+    the team barrier, the slot's loads, the rest."""
+    ms = C.c_float(0)
+    st = (C.c_uint * 12)()
+    _check(lib().turbofft_membench_team(team_blocks, piece_kib, policy, blocks_per_cu, src_ptr, scratch_ptr, scratch_bytes, dst_ptr, nbytes, limit_ms,
+                                        warmup, reps, stream, C.byref(ms), st))
+    return ms.value, {"timed_out": st[0], "waits": st[1], "polls": st[2], "blocks": st[3], "us_per_round": [v / 100.0 for v in list(st)[4:10]],
+                      "rounds_per_block": st[10]}
 
 
 def membench(mode: int, src_ptr: int, dst_ptr: int, nbytes: int, warmup: int = 2, reps: int = 10, stream: int = 0) -> float:
@@ -281,6 +297,21 @@ class TurboFFT:
 
     def set_small_batch(self, enable: bool):
         _check(lib().turbofft_plan_set_small_batch(self._h, int(bool(enable))))
+
+    def set_fused(self, enable: bool):
+        """Switch the plan's fused kernel (both launches of a two-launch plan in one) off or on."""
+        _check(lib().turbofft_plan_set_fused(self._h, int(bool(enable))))
+
+    def fused_info(self):
+        """None when the plan holds no enabled fused kernel, else a dict with its team size, transforms per piece,
+        teams per XCD and grid."""
+        v = [C.c_int(0) for _ in range(4)]
+        rc = lib().turbofft_plan_fused_info(self._h, *[C.byref(x) for x in v])
+        if rc < 0:
+            _check(rc)
+        if rc == 0:
+            return None
+        return {"team_blocks": v[0].value, "transforms_per_piece": v[1].value, "teams_per_xcd": v[2].value, "grid_blocks": v[3].value}
 
     def kernel_names(self) -> List[str]:
         """Kernels the launches of a forward execution run with the current settings."""

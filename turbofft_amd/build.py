@@ -23,7 +23,7 @@ ROOT = os.path.dirname(HERE)
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-from turbofft_amd.codegen.fft_codegen import KernelSpec, collect_keys, generate_source, registry_source  # noqa: E402
+from turbofft_amd.codegen.fft_codegen import KernelSpec, collect_keys, generate_fused_source, generate_source, pair_of_row, registry_source  # noqa: E402
 from turbofft_amd.codegen.plan import load_plan_csv  # noqa: E402
 
 CSRC = os.path.join(HERE, "csrc")
@@ -45,6 +45,23 @@ def ft_override_path(dtype: str, gpu: str = "gfx950") -> str:
 
 def tt_override_path(dtype: str, gpu: str = "gfx950") -> str:
     return os.path.join(HERE, "param", gpu, f"param_{dtype}_tt.csv")
+
+
+def pair_path(dtype: str, gpu: str = "gfx950") -> str:
+    return os.path.join(HERE, "param", gpu, f"param_{dtype}_pair.csv")
+
+
+def all_pairs(extra_csv=()):
+    """Fused pairs: the rows of param_<T>_pair.csv and of extra CSVs given as (dtype, path, "pair")."""
+    pairs = {}
+    for dtype in ("float2", "double2"):
+        paths = [pair_path(dtype)] if os.path.exists(pair_path(dtype)) else []
+        paths += [e[1] for e in extra_csv if e[0] == dtype and len(e) > 2 and e[2] == "pair"]
+        for path in paths:
+            for r in load_plan_csv(path):
+                fs = pair_of_row(r, dtype)
+                pairs.setdefault(fs.name, fs)
+    return list(pairs.values())
 
 
 def all_specs(extra_csv=()):
@@ -71,6 +88,10 @@ def all_specs(extra_csv=()):
         if os.path.exists(small):
             for key in collect_keys([dataclasses.replace(r, tiles=0) for r in load_plan_csv(small)], dtype, [0]):
                 specs.setdefault(key.name, key)
+        # the two launches of a fused pair also exist on their own (the same shapes as two launches)
+        if os.path.exists(pair_path(dtype)):
+            for key in collect_keys(load_plan_csv(pair_path(dtype)), dtype, [0]):
+                specs.setdefault(key.name, key)
         variants = os.path.join(HERE, "param", "gfx950", f"variants_{dtype}.csv")
         if os.path.exists(variants):
             csvs.append((variants, [0, 1]))
@@ -80,7 +101,7 @@ def all_specs(extra_csv=()):
             csvs.append((shapes, [0]))
         for e in extra_csv:
             if e[0] == dtype:
-                csvs.append((e[1], {"noft": [0], "tt": [3]}.get(e[2] if len(e) > 2 else "", [0, 1])))
+                csvs.append((e[1], {"noft": [0], "tt": [3], "pair": [0]}.get(e[2] if len(e) > 2 else "", [0, 1])))
         for path, variants in csvs:
             rows = load_plan_csv(path)
             for key in collect_keys(rows, dtype, variants):
@@ -126,6 +147,14 @@ def builtin_csv_source() -> str:
         out.append(f"    if (datatype == {i}) return\n{lit}        \"\";")
     out.append('    return "";')
     out.append("}")
+    out.append("// two-launch rows that plain plans run as one fused kernel")
+    out.append('extern "C" const char* tfft_builtin_param_pair_csv(int datatype) {')
+    for i, dtype in enumerate(("float2", "double2")):
+        text = open(pair_path(dtype)).read() if os.path.exists(pair_path(dtype)) else ""
+        lit = "".join('        "%s\\n"\n' % ln.replace('"', '\\"') for ln in text.splitlines())
+        out.append(f"    if (datatype == {i}) return\n{lit}        \"\";")
+    out.append('    return "";')
+    out.append("}")
     out.append("// rows of narrow tiles that plain plans run for small batches (column 21: largest batch)")
     out.append('extern "C" const char* tfft_builtin_param_small_csv(int datatype) {')
     for i, dtype in enumerate(("float2", "double2")):
@@ -157,6 +186,7 @@ def build(force: bool = True, jobs: int = 8, extra_csv=(), verbose: bool = True)
     os.makedirs(GEN, exist_ok=True)
     os.makedirs(os.path.dirname(BIN), exist_ok=True)
     specs = all_specs(extra_csv)
+    pairs = all_pairs(extra_csv)
     srcs = []
     wanted = set()
     for sp in specs:
@@ -164,8 +194,13 @@ def build(force: bool = True, jobs: int = 8, extra_csv=(), verbose: bool = True)
         write_if_changed(path, generate_source([sp], False))
         srcs.append(path)
         wanted.add(os.path.basename(path))
+    for fs in pairs:
+        path = os.path.join(GEN, fs.name + ".hip")
+        write_if_changed(path, generate_fused_source(fs, False))
+        srcs.append(path)
+        wanted.add(os.path.basename(path))
     reg = os.path.join(GEN, "tfft_registry.hip")
-    write_if_changed(reg, registry_source(specs))
+    write_if_changed(reg, registry_source(specs, pairs))
     srcs.append(reg)
     wanted.add("tfft_registry.hip")
     bcsv = os.path.join(GEN, "tfft_builtin_param.cpp")
@@ -189,7 +224,7 @@ def build(force: bool = True, jobs: int = 8, extra_csv=(), verbose: bool = True)
         todo.append((s, obj, stale))
     n_stale = sum(1 for t in todo if t[2])
     if verbose:
-        print(f"[turbofft build] {len(specs)} kernels, compiling {n_stale} of {len(todo)} objects with {jobs} jobs", flush=True)
+        print(f"[turbofft build] {len(specs)} kernels and {len(pairs)} fused pairs, compiling {n_stale} of {len(todo)} objects with {jobs} jobs", flush=True)
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         futs = []
         for s, obj, stale in todo:
@@ -210,7 +245,7 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--incremental", action="store_true", help="recompile only what changed")
     ap.add_argument("-j", type=int, default=8)
-    ap.add_argument("--extra", action="append", default=[], metavar="DTYPE:CSV[:noft|:tt]",
+    ap.add_argument("--extra", action="append", default=[], metavar="DTYPE:CSV[:noft|:tt|:pair]",
                     help="also build the kernels needed by another plan CSV (tuning)")
     a = ap.parse_args()
     extra = [tuple(e.split(":")) for e in a.extra]

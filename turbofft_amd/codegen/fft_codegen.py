@@ -207,10 +207,19 @@ class KernelSpec:
 
 
 class KernelEmitter:
-    def __init__(self, spec: KernelSpec, err_smoothing=1000, err_inj=100, err_threshold=1e-3):
+    def __init__(self, spec: KernelSpec, err_smoothing=1000, err_inj=100, err_threshold=1e-3, role: Optional[str] = None,
+                 block_threads: Optional[int] = None):
         self.s = spec
         self.T2 = spec.T2
         self.R = spec.R
+        # Half of a fused pair (one kernel runs both launches of a two-launch plan, the intermediate
+        # staying in a slot that the XCD's L2 holds): "A" writes its tiles into the slot, "B" reads its
+        # tiles from it.  Slot addresses are relative to the first element of the piece the team works
+        # on; `block_threads` is the block size of the fused kernel (a half with fewer threads leaves the
+        # other wavefronts idle between barriers).
+        self.role = role
+        self.block_threads = block_threads or spec.threads
+        self.prefetched = False     # half "A": a member's first tile of a piece arrives in rn[] (fetched during the piece before)
         # Single-launch kernels address global memory through buffer instructions (uniform base
         # in SGPRs, one shared 32-bit lane offset): fewer address registers and no per-access
         # vector arithmetic, +4-5 % on the large tiles.  The strided accesses of the column and
@@ -225,6 +234,10 @@ class KernelEmitter:
             self.GLD += "N"
         if nt & 2:
             self.GST += "N"
+        if role == "A":
+            self.GST = "GSTG"       # the slot is meant to stay in the L2: default policy
+        if role == "B":
+            self.GLD = "GLDUS"      # agent-scope loads: a CU's L1 may still hold the slot's previous contents
         self.TWL, self.TWLU = ("TWLD", "TWLDU") if buf else ("TWLG", "TWLGU")
 
     def pair_access(self) -> bool:
@@ -514,6 +527,8 @@ class KernelEmitter:
             c(f"const long long outer{sfx} = ({tile}) >> tpl{sfx};")
             c(f"const long long ubase{sfx} = (outer{sfx} << ({lNi} + a.log_ncols)) + ((long long)ct{sfx} << {lBS});")
             c(f"const long long gstep{sfx} = {sp.Tr}ll << a.log_ncols;")
+            if self.role == "A":
+                c(f"const long long ubase_st{sfx} = ubase{sfx} - piece_base;")
         else:
             c(f"const unsigned ctl{sfx} = (unsigned)a.logC - {lBS}u;")
             c(f"const unsigned ct{sfx} = (unsigned)(({tile}) & ((1ll << ctl{sfx}) - 1));")
@@ -523,6 +538,8 @@ class KernelEmitter:
             c(f"const unsigned ls{sfx} = (unsigned)a.logN - {lNi}u;")
             c(f"const long long ubase_out{sfx} = tb{sfx} + (ct{sfx} << {lBS}) + ((long long)qd{sfx} << a.logC);")
             c(f"const long long gstep{sfx} = {sp.Tr}ll << ls{sfx};")
+            if self.role == "B":
+                c(f"const long long ubase_ld{sfx} = ubase_in{sfx} - piece_base;")
         names = {"row1": ["row0", "ubase"], "col": ["tpl", "ct", "outer", "ubase", "gstep"],
                  "rowT": ["ctl", "ct", "qd", "tb", "ubase_in", "ls", "ubase_out", "gstep"]}[sp.kind]
         c(" ".join(f"(void){n}{sfx};" for n in names))
@@ -583,7 +600,7 @@ class KernelEmitter:
         else:
             c(f"const unsigned gi{sfx} = ((s << a.logQ) << {lNi}) + x;")
             for e in range(sp.n):
-                c(f"{dst}[{e}] = {self.GLD}(in, ubase_in{sfx}, {sp.Tr * e}, gi{sfx});")
+                c(f"{dst}[{e}] = {self.GLD}(in, {'ubase_ld' if self.role == 'B' else 'ubase_in'}{sfx}, {sp.Tr * e}, gi{sfx});")
         if int(sp.key.inv) and sp.kind in ("row1", "col"):
             # inverse plan, first launch: a forward transform of (im, re) is (im, re) of the
             # inverse one.  A compile-time exchange costs nothing (the loaded register pair is
@@ -641,7 +658,7 @@ class KernelEmitter:
             if sp.dc:
                 self.emit_patch_load(c, [f"{self.GLDC}(out, ubase, {e} * gstep, go)" for e in range(sp.n)])
             for e in range(sp.n):
-                c(f"{self.GST}(out, ubase, {e} * gstep, go, r[{self.out_reg(e)}]);")
+                c(f"{self.GST}(out, {'ubase_st' if self.role == 'A' else 'ubase'}, {e} * gstep, go, r[{self.out_reg(e)}]);")
         else:
             c("const unsigned go = s + (x << ls);")
             if sp.dc:
@@ -995,7 +1012,16 @@ class KernelEmitter:
                     if sp.dc:
                         c("if (!is_redo) {")
                         c.ind += 1
+                    if self.role == "A" and self.prefetched:
+                        c("if (use_rn) {")
+                        for e in range(sp.n):
+                            c(f"    r[{e}] = rn[{e}];")
+                        c("} else {")
+                        c.ind += 1
                     self.emit_load(c)
+                    if self.role == "A" and self.prefetched:
+                        c.ind -= 1
+                        c("}")
                     if sp.dc:
                         c.ind -= 1
                         c("} else {")
@@ -1310,11 +1336,29 @@ class KernelEmitter:
             c("auto& r = ts[tx].r; auto& rn = ts[tx].rn; auto& cvr = ts[tx].cvr; auto& cwr = ts[tx].cwr; auto& sx = ts[tx].sx; auto& sy = ts[tx].sy; auto& fin1 = ts[tx].fin1; auto& fin2 = ts[tx].fin2; auto& fo1 = ts[tx].fo1; auto& fo2 = ts[tx].fo2; auto& tbad = ts[tx].tbad;")
             c("(void)r; (void)rn; (void)cvr; (void)cwr; (void)sx; (void)sy; (void)fin1; (void)fin2; (void)fo1; (void)fo2; (void)tbad;")
         else:
-            c("{")
+            c(f"if (tx < {sp.threads}u) {{" if self.block_threads > sp.threads else "{")
             c.ind += 1
         c(body.rstrip("\n"))
         c.ind -= 1
         c("}")
+
+    def emit_tile_body(self, c: Code, sim: bool, before_last=None, after_first=None):
+        """One tile of a plain kernel: address decode, then the phases with their barriers.  `before_last`
+        and `after_first` emit block-level code ahead of the tile's last phase (the one that stores) and
+        behind its first (the one that loads)."""
+        self.emit_tile_decode(c)
+        phases = self.phases()
+        for i, (sep, ph) in enumerate(phases):
+            if i:
+                if sim:
+                    c(f"// ---- {sep} ----")
+                elif sep == "barrier":
+                    c("__syncthreads();")
+            if before_last and i == len(phases) - 1:
+                before_last()
+            self.thread_block(c, sim, ph)
+            if after_first and i == 0:
+                after_first()
 
     def emit_tl_verdict(self, c: Code, sim: bool):
         """Thread-level verification, behind the barrier that follows a tile's last pass: did any thread of the
@@ -1468,6 +1512,205 @@ FILE_HEADER = """// GENERATED by turbofft_amd/codegen/fft_codegen.py -- do not e
 """
 
 
+@dataclass
+class FusedSpec:
+    """Both launches of a two-launch plan as one kernel: a team of blocks on one XCD runs the column
+    launch of a piece (a few whole transforms) into a slot that the XCD's L2 holds, meets, and runs
+    the row launch out of the slot, so the intermediate of the plan never travels to memory."""
+    a: KernelKey       # the column launch (kind "col")
+    b: KernelKey       # the row launch with the transposed store (kind "rowT")
+
+    def __post_init__(self):
+        for k in (self.a, self.b):
+            if int(k.ft) or k.pf or k.xl or k.inv or k.ck or k.wv:
+                raise ValueError(f"{k}: a fused pair is made of plain forward kernels without prefetch or a register budget")
+        if self.a.kind != "col" or self.b.kind != "rowT" or self.a.dtype != self.b.dtype:
+            raise ValueError("a fused pair is a column launch followed by a row launch of the same type")
+        self.sa = KernelSpec(self.a)
+        self.sb = KernelSpec(self.b)
+        self.T2, self.R = self.sa.T2, self.sa.R
+        self.threads = max(self.sa.threads, self.sb.threads)
+        self.lds_bytes = max(self.sa.lds_bytes, self.sb.lds_bytes)
+        self.n = max(self.sa.n, self.sb.n)
+
+    @property
+    def name(self) -> str:
+        t = "f32" if self.a.dtype == "float2" else "f64"
+        a, b = self.a, self.b
+        return (f"tfft_{t}_pair_N{a.logNi}x{b.logNi}_b{a.BS}x{b.BS}_n{a.n}x{b.n}"
+                + (f"_s{int(a.split)}{int(b.split)}" if a.split or b.split else "") + (f"_t{int(a.nt)}{int(b.nt)}" if a.nt or b.nt else ""))
+
+
+def emit_fused(fs: FusedSpec, sim: bool) -> str:
+    c = Code()
+    T2 = fs.T2
+    ea = KernelEmitter(fs.sa, role="A", block_threads=fs.threads)
+    eb = KernelEmitter(fs.sb, role="B", block_threads=fs.threads)
+    ea.prefetched = True
+    prof = bool(os.environ.get("TFFT_PAIR_PROFILE")) and not sim     # diagnostic build: time per part of a round, per block
+
+    def tick(k: int):
+        if prof:
+            c(f"if (f.prof) {{ const long long now_ = (long long)wall_clock64(); pt[{k}] += now_ - pt_last; pt_last = now_; }}")
+    c(f"// {fs.name}: column launch (Ni={fs.sa.Ni}, BS={fs.sa.BS}, n={fs.sa.n}, {fs.sa.threads} threads) and row launch")
+    c(f"// (Ni={fs.sb.Ni}, BS={fs.sb.BS}, n={fs.sb.n}, {fs.sb.threads} threads) of a two-launch plan in one kernel, {fs.threads} threads, LDS {fs.lds_bytes} B")
+
+    def scope(e: KernelEmitter, kargs: str, src: str, dst: Optional[str]):
+        sp = e.s
+        c(f"const tfft_kargs& a = {kargs};")
+        c(f"const {T2}* in = {src};" + (f" {T2}* out = {dst};" if dst else ""))
+        c(f"const {T2}* twhi = (const {T2}*)a.tw_hi; const {T2}* twlo = (const {T2}*)a.tw_lo; (void)twhi; (void)twlo;")
+        LT = fs.R if sp.split else T2
+        if sim:
+            c(f"std::vector<{LT}> ldsv({sp.lds_elems}); {LT}* lds = ldsv.data(); const long long lds_limit = {sp.lds_elems}; (void)lds; (void)lds_limit;")
+            c("const long long twhi_limit = limits[3], twlo_limit = limits[4]; (void)twhi_limit; (void)twlo_limit;")
+            if e.role == "A":
+                c("const long long in_limit = limits[0], out_limit = f.piece_elems; (void)in_limit; (void)out_limit;")
+            else:
+                c("const long long in_limit = f.piece_elems, out_limit = limits[1]; (void)in_limit; (void)out_limit;")
+        else:
+            c(f"{LT}* lds = ({LT}*)lds_raw; (void)lds;")
+
+    def prefetch(piece: str, member: str):
+        """A member's first column tile of `piece` into rn[]: issued while the member still works on the piece
+        before, so that the latency of memory is spent behind that work."""
+        c("{")
+        c.ind += 1
+        scope(ea, "a0", "in_g", None)
+        c(f"const long long piece_base = ({piece}) * f.piece_elems; (void)piece_base;")
+        c(f"const long long tile_n = ({piece}) * f.tiles_a + {member};")
+        c(f"if ({member} < f.tiles_a && tile_n < a.ntiles) {{")
+        c.ind += 1
+        ea.emit_tile_decode(c, "tile_n", "_n")
+        pre = Code()
+        ea.map_vars(pre, 0)
+        ea.emit_load(pre, "rn", "_n")
+        ea.thread_block(c, sim, pre.text())
+        c.ind -= 1
+        c("}")
+        c.ind -= 1
+        c("}")
+
+    def half(e: KernelEmitter, kargs: str, tiles: str, src: str, dst: str, member: str, before_last=None, after_first=None):
+        c("{")
+        c.ind += 1
+        scope(e, kargs, src, dst)
+        c(f"for (long long j = {member}; j < {tiles}; j += f.team) {{")
+        c.ind += 1
+        c(f"const long long tile = piece * {tiles} + j;")
+        c("if (tile >= a.ntiles) break;")
+        c(f"const bool use_rn = j == {member}; (void)use_rn;")
+        e.emit_tile_body(c, sim, before_last, after_first)
+        c.ind -= 1
+        c("}")
+        c.ind -= 1
+        c("}")
+
+    if sim:
+        # one team and one slot, its members one after the other: the index algebra and the slot's bounds
+        c(f'extern "C" void {fs.name}_sim(const {T2}* in_g, {T2}* out_g, const {T2}* tw, const tfft_kargs* a0p, const tfft_kargs* a1p,')
+        c(f"        const tfft_fuse_args* fp, {T2}* slot, const long long* limits)")
+        c("{")
+        c.ind += 1
+        c("const tfft_kargs a0 = *a0p, a1 = *a1p; const tfft_fuse_args f = *fp;")
+        c("const long long tw_limit = limits[2]; (void)tw_limit;")
+        c(f"struct TS {{ {T2} r[{fs.n}]; {T2} rn[{fs.n}]; {T2} sh[{fs.n}]; {T2} cvr[{fs.n}]; unsigned cwr[{fs.n}]; {T2} sx[{fs.n}]; {T2} sy[{fs.n}]; {fs.R} fin1, fin2, fo1, fo2; bool tbad; }};")
+        c(f"std::vector<TS> ts({fs.threads}); for (auto& z : ts) z = TS();")
+        c("for (long long piece = 0; piece < f.npieces; ++piece) {")
+        c.ind += 1
+        c("const long long piece_base = piece * f.piece_elems;")
+        c("for (long long member = 0; member < f.team; ++member) {")
+        c.ind += 1
+        prefetch("piece", "member")
+        half(ea, "a0", "f.tiles_a", "in_g", "slot", "member")
+        c.ind -= 1
+        c("}")
+        c("for (long long member = 0; member < f.team; ++member)")
+        half(eb, "a1", "f.tiles_b", "slot", "out_g", "member")
+        c.ind -= 1
+        c("}")
+        c.ind -= 1
+        c("}")
+        return c.text()
+    c(f'extern "C" __global__ __launch_bounds__({fs.threads})')
+    c(f"void {fs.name}(const {T2}* __restrict__ in_g, {T2}* __restrict__ out_g, const {T2}* __restrict__ tw, const tfft_kargs a0, const tfft_kargs a1, const tfft_fuse_args f)")
+    c("{")
+    c.ind += 1
+    c("extern __shared__ __align__(16) unsigned char lds_raw[];")
+    c("__shared__ unsigned team_words[4];")
+    c("const unsigned tx = threadIdx.x;")
+    c(f"{T2} r[{fs.n}];")
+    c(f"{T2} rn[{fs.sa.n}];")
+    c("tfft_team tm;")
+    c("if (tfft_team_join(f, tm, team_words)) {")
+    c.ind += 1
+    c(f"{T2}* const slot = ({T2}*)f.slots + (long long)tm.slot * f.piece_elems;")
+    c("const long long member = (long long)tm.member;")
+    c("long long piece = tfft_team_first(f, tm, team_words);")
+    c("if (piece >= 0)")
+    prefetch("piece", "member")
+    if prof:
+        c("long long pt[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long pt_last = (long long)wall_clock64();")
+    c("for (unsigned round = 0; piece >= 0; ++round) {")
+    c.ind += 1
+    c("const long long piece_base = piece * f.piece_elems;")
+
+    def slot_free():
+        # the tile's last phase stores into the slot: not before every member has read what the round before left there
+        tick(0)
+        c("if (use_rn && round && !tfft_team_free(f, tm, round, team_words)) goto tfft_out;")
+        tick(3)
+
+    half(ea, "a0", "f.tiles_a", "in_g", "slot", "member", before_last=slot_free)
+    # every member's part of the slot is in the L2 before any member reads a row of it
+    c("long long next = -1;")
+    tick(0)
+    c("if (!tfft_team_meet(f, tm, round, team_words, next)) goto tfft_out;")
+    tick(1)
+    c("bool fetched = false;")
+
+    def fetch_next():
+        # behind the loads of this member's first row tile: its first column tile of the next piece
+        tick(5)
+        c("if (!fetched && next >= 0) {")
+        c.ind += 1
+        prefetch("next", "member")
+        c("fetched = true;")
+        c.ind -= 1
+        c("}")
+        tick(6)
+
+    half(eb, "a1", "f.tiles_b", "slot", "out_g", "member", after_first=fetch_next)
+    fetch_next()
+    c("tfft_team_release(tm);")
+    tick(2)
+    if prof:
+        c("pt[4] += 1;")
+    c("piece = next;")
+    c.ind -= 1
+    c("}")
+    if prof:
+        c("if (f.prof && tx == 0) for (int k = 0; k < 8; ++k) f.prof[8 * (size_t)blockIdx.x + k] = (unsigned long long)pt[k];")
+        c.ind -= 1
+        c("}")
+        c("tfft_out:")
+    else:
+        c.ind -= 1
+        c("}")
+        c("tfft_out:")
+    c("tfft_team_leave(f, team_words);")
+    c.ind -= 1
+    c("}")
+    return c.text()
+
+
+def generate_fused_source(fs: FusedSpec, sim: bool) -> str:
+    head = FILE_HEADER
+    if sim:
+        head = FILE_HEADER.replace('#include "../tfft_device.h"', '#define TFFT_SIM 1\n#include "../tfft_device.h"')
+    return head + "\n" + emit_fused(fs, sim)
+
+
 def generate_source(specs: Sequence[KernelSpec], sim: bool) -> str:
     out = [FILE_HEADER]
     if sim:
@@ -1477,7 +1720,7 @@ def generate_source(specs: Sequence[KernelSpec], sim: bool) -> str:
     return "\n".join(out)
 
 
-def registry_source(specs: Sequence[KernelSpec]) -> str:
+def registry_source(specs: Sequence[KernelSpec], pairs: Sequence["FusedSpec"] = ()) -> str:
     """C table the host driver uses to find a kernel for a launch
     (the role of TurboFFT_Kernel_Entry, include/TurboFFT.h:22-25,118-526)."""
     c = Code()
@@ -1496,7 +1739,29 @@ def registry_source(specs: Sequence[KernelSpec]) -> str:
     c("    *count = (int)(sizeof(tfft_kernel_table_) / sizeof(tfft_kernel_table_[0]));")
     c("    return tfft_kernel_table_;")
     c("}")
+    for fs in pairs:
+        c(f'extern "C" __global__ void {fs.name}(const {fs.T2}*, {fs.T2}*, const {fs.T2}*, const tfft_kargs, const tfft_kargs, const tfft_fuse_args);')
+    c("static const tfft_pair_entry tfft_pair_table_[] = {")
+    for fs in pairs:
+        a, b = fs.a, fs.b
+        c(f'    {{"{fs.name}", (const void*){fs.name}, {0 if a.dtype == "float2" else 1}, {a.logNi}, {a.BS}, {a.n}, {int(a.split)}, {int(a.nt)}, '
+          f'{b.logNi}, {b.BS}, {b.n}, {int(b.split)}, {int(b.nt)}, {fs.threads}, {fs.lds_bytes}}},')
+    c('    {nullptr, nullptr, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0},')
+    c("};")
+    c('extern "C" const tfft_pair_entry* tfft_pair_table(int* count) {')
+    c("    *count = (int)(sizeof(tfft_pair_table_) / sizeof(tfft_pair_table_[0])) - 1;")
+    c("    return tfft_pair_table_;")
+    c("}")
     return c.text()
+
+
+def pair_of_row(row: PlanRow, dtype: str) -> "FusedSpec":
+    """The fused pair of a two-launch row: tile shapes and exchange forms are the row's, the column half
+    keeps the load policy bit and the row half the store policy bit (the slot side of each is fixed)."""
+    if row.launches != 2:
+        raise ValueError(f"row {row.logN}: a fused pair needs a two-launch row")
+    return FusedSpec(KernelKey(dtype, "col", row.logNi[0], row.BS[0], row.n[0], 0, int(row.split[0]) if row.split else 0, 0, 0, 0, (int(row.nt[0]) & 1) if row.nt else 0),
+                     KernelKey(dtype, "rowT", row.logNi[1], row.BS[1], row.n[1], 0, int(row.split[1]) if row.split else 0, 0, 0, 0, (int(row.nt[1]) & 2) if row.nt else 0))
 
 
 def collect_keys(rows: Sequence[PlanRow], dtype: str, ft_variants: Sequence[int], inverse: bool = False) -> List[KernelKey]:

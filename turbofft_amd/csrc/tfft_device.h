@@ -73,6 +73,9 @@ __device__ __forceinline__ void tfft_bst2(float2* p, unsigned voff, unsigned sof
 // the tables in the caches
 #define GLDUN(p, ub, uo, off) tfft_bld<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
 #define GSTUN(p, ub, uo, off, v) tfft_bst<2>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p), (v))
+// agent-scope load (sc1): served by the XCD's L2, never by the CU's own L1 -- for data that blocks on
+// other CUs of the XCD wrote during this kernel
+#define GLDUS(p, ub, uo, off) tfft_bld<16>((p) + (ub), (unsigned)(off) * TFFT_ESZ(p), (unsigned)(uo) * TFFT_ESZ(p))
 // plain global-pointer forms of the same accesses
 #define GLDG(p, ub, uo, off) (((p) + ((ub) + (uo)))[(off)])
 #define GSTG(p, ub, uo, off, v) (((p) + ((ub) + (uo)))[(off)] = (v))
@@ -137,6 +140,136 @@ __device__ __forceinline__ long long tfft_uni(long long v) {
 // thread-level verification: one word per wavefront at byte `off` of the block's LDS says whether any of
 // its lanes objected to the tile (a wave vote, then lane 0 writes); the block reads the words behind a barrier
 #define TL_VOTE(off, bad) { const int wany_ = __any((bad) ? 1 : 0); if ((tx & 63u) == 0u) ((unsigned*)(lds_raw + (off)))[tx >> 6] = wany_ ? 1u : 0u; }
+
+// ---- teams of a fused pair (tfft_fuse_args) ----
+// A team is `team` blocks that arrived one after the other on one XCD; its first member is its leader.
+// Every wait is thread 0's, on an agent-scope counter, and bounded: after limit_ms the waiting block sets
+// the give-up word, which every other wait reads on each eighth poll, and all blocks leave.  What orders
+// the slot's data: a block waits until its own stores are acknowledged (they are in the L2 then) before it
+// counts itself in, and the readers use agent-scope loads.
+// The leader names pieces two rounds ahead (word r % 2 of the pair holds round r's name, tagged r + 1):
+// when a member leaves the meeting of round r the name of round r + 1 has long been there, so it can
+// start fetching that piece while it still works on this one.
+struct tfft_team { unsigned slot, member, xcc, index; unsigned* a; unsigned* b; unsigned long long* cur; long long t_limit; };
+
+__device__ __forceinline__ bool tfft_team_give_up(const tfft_fuse_args& f, long long t_limit, unsigned polls) {
+    if ((polls & 7u) != 7u) return false;
+    if (tfft_ps_load(&f.ctl[0])) return true;
+    if ((long long)wall_clock64() > t_limit) {
+        atomicExch(&f.ctl[0], 1u);
+        if (f.err_host) __hip_atomic_store(f.err_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        return true;
+    }
+    return false;
+}
+// thread 0: until *p >= k
+__device__ __forceinline__ bool tfft_team_wait(unsigned* p, unsigned k, const tfft_fuse_args& f, long long t_limit) {
+    for (unsigned polls = 0;; ++polls) {
+        if (tfft_ps_load(p) >= k) return true;
+        if (tfft_team_give_up(f, t_limit, polls)) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+// thread 0: the name of `round` (piece + 1, 0: none), 0 also when the wait gave up
+__device__ __forceinline__ unsigned tfft_team_name(const tfft_fuse_args& f, const tfft_team& tm, unsigned round) {
+    for (unsigned polls = 0;; ++polls) {
+        const unsigned long long v = tfft_ps_load(tm.cur + 16 * (round & 1u));
+        if ((unsigned)(v >> 32) == round + 1u) return (unsigned)v;
+        if (tfft_team_give_up(f, tm.t_limit, polls)) return 0u;
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+// thread 0 of the leader: take a piece off the queue and name it for `round`
+__device__ __forceinline__ void tfft_team_claim(const tfft_fuse_args& f, const tfft_team& tm, unsigned round, bool take) {
+    unsigned p1 = 0;
+    if (take) { const unsigned p = atomicAdd(&f.ctl[32], 1u); p1 = (long long)p < f.npieces ? p + 1u : 0u; }
+    tfft_ps_store(tm.cur + 16 * (round & 1u), ((unsigned long long)(round + 1u) << 32) | p1);
+}
+// false: this block has no team (its XCD's teams were full when it arrived)
+__device__ __forceinline__ bool tfft_team_join(const tfft_fuse_args& f, tfft_team& tm, unsigned* w) {
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;      // XCC_ID[3:0] of the hardware register
+    if (threadIdx.x == 0) w[0] = atomicAdd(&f.ctl[96 + 32 * xcc], 1u);
+    __syncthreads();
+    const unsigned idx = tfft_uni(w[0]);
+    __syncthreads();
+    const unsigned team = idx / (unsigned)f.team;
+    tm.xcc = xcc; tm.index = team; tm.member = idx % (unsigned)f.team;
+    tm.slot = xcc * (unsigned)f.teams_per_xcd + team;
+    unsigned* base = f.ctl + 352 + 128 * (size_t)tm.slot;
+    tm.a = base; tm.b = base + 32; tm.cur = (unsigned long long*)(base + 64);
+    tm.t_limit = (long long)wall_clock64() + (long long)f.limit_ms * 100000ll;   // 100 MHz counter
+    return team < (unsigned)f.teams_per_xcd;
+}
+// The team's first piece, or -1 when there is none.  The leader waits until the team is complete -- or the queue
+// empty: then a team that forms late has nothing to do -- and names rounds 0 and 1.
+__device__ __forceinline__ long long tfft_team_first(const tfft_fuse_args& f, const tfft_team& tm, unsigned* w) {
+    if (threadIdx.x == 0) {
+        bool ok = true;
+        if (tm.member == 0) {
+            bool complete = false;
+            for (unsigned polls = 0;; ++polls) {
+                if (tfft_ps_load(&f.ctl[96 + 32 * tm.xcc]) >= (tm.index + 1u) * (unsigned)f.team) { complete = true; break; }
+                if ((long long)tfft_ps_load(&f.ctl[32]) >= f.npieces) break;
+                if (tfft_team_give_up(f, tm.t_limit, polls)) { ok = false; break; }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (ok) { tfft_team_claim(f, tm, 0u, complete); tfft_team_claim(f, tm, 1u, complete); }
+        }
+        w[1] = ok ? tfft_team_name(f, tm, 0u) : 0u;
+    }
+    __syncthreads();
+    const unsigned name = tfft_uni(w[1]);
+    __syncthreads();
+    return (long long)name - 1;
+}
+// Between the two launches of a piece: every member's tiles are in the slot.  `next` is the piece of the next
+// round (-1: none).  The leader, once every member has arrived (all have read this round's name by then, whose
+// word is the one written now), names the round after the next.
+__device__ __forceinline__ bool tfft_team_meet(const tfft_fuse_args& f, const tfft_team& tm, unsigned round, unsigned* w, long long& next) {
+    TFFT_WAIT_VMEM();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        atomicAdd(tm.a, 1u);
+        const bool ok = tfft_team_wait(tm.a, (unsigned)f.team * (round + 1u), f, tm.t_limit);
+        unsigned name = 0;
+        if (ok) {
+            name = tfft_team_name(f, tm, round + 1u);
+            if (tm.member == 0) tfft_team_claim(f, tm, round + 2u, name != 0u);
+        }
+        w[1] = name;
+        w[2] = ok ? 1u : 0u;
+    }
+    __syncthreads();
+    const unsigned ok = tfft_uni(w[2]), name = tfft_uni(w[1]);
+    __syncthreads();
+    next = (long long)name - 1;
+    return ok != 0u;
+}
+// before a member's first store of `round` (> 0) into the slot: every member has finished reading what the
+// round before left there
+__device__ __forceinline__ bool tfft_team_free(const tfft_fuse_args& f, const tfft_team& tm, unsigned round, unsigned* w) {
+    if (threadIdx.x == 0) w[2] = tfft_team_wait(tm.b, (unsigned)f.team * round, f, tm.t_limit) ? 1u : 0u;
+    __syncthreads();
+    const unsigned ok = tfft_uni(w[2]);
+    __syncthreads();
+    return ok != 0u;
+}
+// after the row launch of a piece: this member no longer reads the slot (what it loaded from the slot has been
+// computed with, so those loads have returned; its stores to memory are nobody's business here)
+__device__ __forceinline__ void tfft_team_release(const tfft_team& tm) {
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(tm.b, 1u);
+}
+// every block of the grid, last thing: the last one to leave clears the control block for the next launch
+__device__ __forceinline__ void tfft_team_leave(const tfft_fuse_args& f, unsigned* w) {
+    __syncthreads();
+    if (threadIdx.x == 0) w[3] = atomicAdd(&f.ctl[64], 1u) == gridDim.x - 1u ? 1u : 0u;
+    __syncthreads();
+    if (w[3]) {
+        const unsigned words = 352u + 128u * 8u * (unsigned)f.teams_per_xcd;
+        for (unsigned i = threadIdx.x; i < words; i += blockDim.x) tfft_ps_store(&f.ctl[i], 0u);
+    }
+}
 #else
 #include <cmath>
 #include <cstdio>
@@ -159,6 +292,7 @@ extern long long tfft_sim_errors;
 #define GLDG(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTG(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
 #define GLDUN(p, ub, uo, off) GLDU(p, ub, uo, off)
+#define GLDUS(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTUN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)
 #define GLDGN(p, ub, uo, off) GLDU(p, ub, uo, off)
 #define GSTGN(p, ub, uo, off, v) GSTU(p, ub, uo, off, v)

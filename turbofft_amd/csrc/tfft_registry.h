@@ -23,7 +23,23 @@ typedef struct tfft_kernel_entry {
     int lds_bytes;       // dynamic LDS
 } tfft_kernel_entry;
 
+// A fused pair: the column launch and the row launch of a two-launch plan as one kernel
+// (arguments: in, out, twiddles, the two launches' tfft_kargs, tfft_fuse_args).
+typedef struct tfft_pair_entry {
+    const char* name;
+    const void* func;
+    int datatype;
+    int logN1, BS1, n1, split1, nt1;    // the column launch (nt1: bit 0 only, its loads)
+    int logN2, BS2, n2, split2, nt2;    // the row launch (nt2: bit 1 only, its stores)
+    int threads;                        // block size (the larger of the two halves)
+    int lds_bytes;                      // dynamic LDS (the larger of the two halves)
+} tfft_pair_entry;
+
 #ifdef __cplusplus
-extern "C"
+extern "C" {
 #endif
 const tfft_kernel_entry* tfft_kernel_table(int* count);
+const tfft_pair_entry* tfft_pair_table(int* count);
+#ifdef __cplusplus
+}
+#endif

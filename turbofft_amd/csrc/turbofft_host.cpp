@@ -24,6 +24,7 @@
 extern "C" const char* tfft_builtin_param_csv(int datatype);   // generated: the gfx950 CSV text
 extern "C" const char* tfft_builtin_param_ft_csv(int datatype);   // generated: rows replaced in FT plans
 extern "C" const char* tfft_builtin_param_tt_csv(int datatype);   // generated: rows replaced in plans with thread-level verification
+extern "C" const char* tfft_builtin_param_pair_csv(int datatype);   // generated: two-launch rows that run as one fused kernel
 extern "C" const char* tfft_builtin_param_small_csv(int datatype);   // generated: rows for batches too small to fill the device
 
 namespace {
@@ -76,6 +77,8 @@ constexpr long long kPartTickets = 1ll << 20;
 constexpr int kCuLdsBytes = 160 * 1024;     // LDS of one gfx950 compute unit
 constexpr long long kFixGrid = 256;         // blocks of the launch that recomputes queued tiles
 constexpr size_t kMaxSmallWs = 8;           // intermediate buffers (one per stream) a plan keeps for its small-batch row
+constexpr size_t kMaxPairWs = 8;            // slot sets (one per stream) a plan keeps for its fused pair
+constexpr int kPairLimitMs = 2000;          // longest wait of a block of a fused pair for other blocks
 // smallest err_threshold the compact checksum tables serve: half-precision entries (fp32 kernels)
 // leave up to 1e-4 of the checksum magnitude as residual on clean data, single-precision ones
 // (fp64 kernels) 1e-8
@@ -83,7 +86,7 @@ constexpr double kCompactMinThreshold32 = 5e-4, kCompactMinThreshold64 = 1e-6;
 constexpr double kSqrt3_2_literal = 0.8660253882408142;   // abft.h:22-28, float-rounded
 
 struct Row {
-    int v[36];           // 11 reference columns + optional per-launch flags: split exchange,
+    int v[40];           // 11 reference columns + optional per-launch flags: split exchange,
                          // prefetch, cross-lane last pass; then the tiles-per-block hint, the
                          // per-launch wavefronts-per-SIMD the plain kernel was compiled for and
                          // the per-launch non-temporal access bits, then the per-launch
@@ -91,6 +94,11 @@ struct Row {
                          // compact-checksum-table flag of the fault-tolerant kernel, then the per-launch
                          // number of tiles a block walks of a checksum group that several blocks share
                          // (0 = the library's default)
+    // rows of fused pairs (columns 37-39): blocks per team (0: 8), transforms per piece (0: 1), teams per XCD
+    // (0: as many as one block per CU gives)
+    int team() const { return v[36] > 0 ? v[36] : 8; }
+    int per_piece() const { return v[37] > 0 ? v[37] : 1; }
+    int teams() const { return v[38]; }
     int ck(int i) const { return v[30 + i]; }
     int gp(int i) const { return v[33 + i]; }
     int nt(int i) const { return v[24 + i]; }
@@ -118,7 +126,7 @@ bool parse_csv(std::istream& in, std::vector<Row>& rows) {
         std::istringstream ls(line);
         std::string tok;
         int c = 0;
-        while (c < 36 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
+        while (c < 40 && std::getline(ls, tok, ',')) r.v[c++] = atoi(tok.c_str());
         if (c < 11) return false;
         rows.push_back(r);
     }
@@ -136,6 +144,17 @@ const tfft_kernel_entry* find_kernel(int datatype, int kind, int logNi, int BS, 
     for (int i = 0; i < cnt; ++i)
         if (t[i].datatype == datatype && t[i].kind == kind && t[i].logNi == logNi && t[i].BS == BS &&
             t[i].n == n && t[i].ft == ft && t[i].split == split && t[i].pf == pf && t[i].xl == xl && t[i].wv == wv && t[i].nt == nt && t[i].inv == inv && t[i].ck == ck)
+            return &t[i];
+    return nullptr;
+}
+
+const tfft_pair_entry* find_pair(int datatype, const Row& r) {
+    int cnt = 0;
+    const tfft_pair_entry* t = tfft_pair_table(&cnt);
+    for (int i = 0; i < cnt; ++i)
+        if (t[i].datatype == datatype && t[i].logN1 == r.logNi(0) && t[i].BS1 == r.BS(0) && t[i].n1 == r.n(0) && t[i].split1 == (r.split(0) ? 1 : 0) &&
+            t[i].nt1 == (r.nt(0) & 1) && t[i].logN2 == r.logNi(1) && t[i].BS2 == r.BS(1) && t[i].n2 == r.n(1) && t[i].split2 == (r.split(1) ? 1 : 0) &&
+            t[i].nt2 == (r.nt(1) & 2))
             return &t[i];
     return nullptr;
 }
@@ -267,6 +286,17 @@ struct turbofft_plan {
     std::vector<SmallWs> small_ws;
     std::mutex small_mu;
     bool small_enabled = true;
+    // Fused pair (plain built-in two-launch plans): a row whose two launches run as ONE kernel, the
+    // intermediate staying in slots that the XCDs' L2s hold.  `pair` is a plan of its own for that row
+    // (tables, launch geometry); the fields below it are set on that plan.  Every stream that has run
+    // the pair owns a set of slots and a control block, so executions on different streams share none.
+    turbofft_plan* pair = nullptr;
+    const tfft_pair_entry* pk = nullptr;
+    int pair_team = 0, pair_per_piece = 0, pair_grid = 0, pair_teams_per_xcd = 0, pair_limit_ms = kPairLimitMs;
+    struct PairWs { void* stream; bool assigned; void* slots; unsigned* ctl; unsigned* err_host; };
+    std::vector<PairWs> pair_ws;
+    std::mutex pair_mu;
+    bool pair_enabled = true;
     bool compact_enabled = true;      // TURBOFFT_COMPACT_CHECKSUM=0 keeps the full-table kernels
 };
 
@@ -328,6 +358,12 @@ const char* turbofft_kernel_name(int i) {
 void turbofft_plan_destroy(turbofft_plan_t* p) {
     if (!p) return;
     if (p->small) turbofft_plan_destroy(p->small);
+    if (p->pair) turbofft_plan_destroy(p->pair);
+    for (auto& w : p->pair_ws) {
+        if (w.slots) (void)hipFree(w.slots);
+        if (w.ctl) (void)hipFree(w.ctl);
+        if (w.err_host) (void)hipHostFree(w.err_host);
+    }
     for (auto& w : p->small_ws) if (w.buf) (void)hipFree(w.buf);
     if (p->tw) (void)hipFree(p->tw);
     for (int i = 0; i < 3; ++i) {
@@ -393,6 +429,27 @@ namespace { int static_workspace(void** ptr); }
 
 static int plan_build_row(turbofft_plan* p, const Row& row);
 
+// One more set of slots and a control block for the fused pair of plan `p` (`q` is the pair's own plan).
+// False when the memory cannot be had; nothing is kept then.
+static bool pair_add_ws(turbofft_plan* p, const turbofft_plan* q, void* stream, bool assigned) {
+    const size_t nslots = (size_t)8 * q->pair_teams_per_xcd;
+    const size_t slot_bytes = ((size_t)q->pair_per_piece << q->logN) * q->esize;
+    const size_t ctl_bytes = sizeof(unsigned) * TFFT_FUSE_CTL_WORDS(nslots);
+    void *sl = nullptr, *ctl = nullptr, *eh = nullptr;
+    bool ok = hipMalloc(&sl, nslots * slot_bytes) == hipSuccess && hipMalloc(&ctl, ctl_bytes) == hipSuccess &&
+              hipHostMalloc(&eh, 64, hipHostMallocDefault) == hipSuccess && hipMemset(ctl, 0, ctl_bytes) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        if (sl) (void)hipFree(sl);
+        if (ctl) (void)hipFree(ctl);
+        if (eh) (void)hipHostFree(eh);
+        return false;
+    }
+    *(volatile unsigned*)eh = 0u;
+    p->pair_ws.push_back({stream, assigned, sl, (unsigned*)ctl, (unsigned*)eh});
+    return true;
+}
+
 static int plan_build(turbofft_plan* p, const char* param_csv) {
     std::vector<Row> rows;
     if (param_csv) {
@@ -445,6 +502,55 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
                 HIP_TRY(hipMalloc(&buf, ((size_t)p->small_max_bs << p->logN) * p->esize));
                 p->small_ws.push_back({nullptr, false, buf});
             }
+            break;
+        }
+    }
+    // (measured at parity with the two launches at best, so a plan holds it only when asked to: TURBOFFT_FUSED=1)
+    const char* fenv = getenv("TURBOFFT_FUSED");
+    if (!param_csv && !p->if_ft && fenv && atoi(fenv) == 1) {
+        // the row whose two launches run as one kernel, if the built-in table has one for this size
+        std::vector<Row> pairs;
+        if (const char* pcsv = getenv("TURBOFFT_FUSED_CSV")) {
+            // tuning aid: another table of fused rows (its kernels must have been built: build.py --extra <type>:<csv>:pair)
+            std::ifstream pf(pcsv);
+            if (!pf.is_open() || !parse_csv(pf, pairs)) return fail(TURBOFFT_ENOPLAN, "cannot read the fused-pair table %s", pcsv);
+        } else {
+            std::istringstream pin(tfft_builtin_param_pair_csv(p->datatype));
+            if (!parse_csv(pin, pairs)) return fail(TURBOFFT_ENOPLAN, "built-in fused-pair plan table is malformed");
+        }
+        for (const Row& pr : pairs) {
+            if (pr.logN() != p->logN || pr.launches() != 2) continue;
+            const tfft_pair_entry* pk = find_pair(p->datatype, pr);
+            if (!pk) return fail(TURBOFFT_ENOPLAN, "no compiled fused pair for logN=%d", p->logN);
+            turbofft_plan* q = new turbofft_plan();
+            q->logN = p->logN; q->datatype = p->datatype; q->thread_bs = 1; q->xcd_chunk = p->xcd_chunk;
+            Row clean = pr;
+            clean.v[20] = 0;
+            rc = plan_build_row(q, clean);
+            if (rc) { turbofft_plan_destroy(q); return rc; }
+            int dev = 0, occ = 0;
+            hipDeviceProp_t prop;
+            if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) { (void)hipGetLastError(); turbofft_plan_destroy(q); return fail(TURBOFFT_EHIP, "cannot query the device"); }
+            if (pk->lds_bytes > kCuLdsBytes) { turbofft_plan_destroy(q); return fail(TURBOFFT_ENOPLAN, "fused pair %s needs %d B of LDS", pk->name, pk->lds_bytes); }
+            if ((size_t)pk->lds_bytes > (size_t)prop.sharedMemPerBlock &&
+                hipFuncSetAttribute(pk->func, hipFuncAttributeMaxDynamicSharedMemorySize, pk->lds_bytes) != hipSuccess) {
+                (void)hipGetLastError(); turbofft_plan_destroy(q); return fail(TURBOFFT_EHIP, "cannot opt %s into %d B of LDS", pk->name, pk->lds_bytes);
+            }
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, pk->func, pk->threads, pk->lds_bytes) != hipSuccess || occ < 1) {
+                (void)hipGetLastError(); turbofft_plan_destroy(q); return fail(TURBOFFT_ENOPLAN, "fused pair %s does not fit on a CU", pk->name);
+            }
+            // every block of the grid has to be resident at once (blocks wait for their team): the row's number of
+            // teams on each of the 8 XCDs, at most what fits there
+            q->pk = pk;
+            q->pair_team = pr.team();
+            q->pair_per_piece = pr.per_piece();
+            const int cus_per_xcd = prop.multiProcessorCount / 8, fit = cus_per_xcd * occ / q->pair_team;
+            q->pair_teams_per_xcd = pr.teams() > 0 ? (pr.teams() < fit ? pr.teams() : fit) : cus_per_xcd / q->pair_team;
+            q->pair_grid = 8 * q->pair_teams_per_xcd * q->pair_team;
+            if (const char* e = getenv("TURBOFFT_FUSED_LIMIT_MS")) if (atoi(e) > 0) q->pair_limit_ms = atoi(e);
+            if (q->pair_teams_per_xcd < 1 || q->pair_teams_per_xcd > 64) { turbofft_plan_destroy(q); break; }   // no room for a team: the plan keeps its two launches
+            p->pair = q;
+            if (!pair_add_ws(p, q, nullptr, false)) { turbofft_plan_destroy(q); p->pair = nullptr; return fail(TURBOFFT_ENOMEM, "no memory for the slots of the fused pair"); }
             break;
         }
     }
@@ -860,6 +966,7 @@ struct exec_opts {
     bool sync_each = false;       // wait for every launch before issuing the next (the reference's timing loop)
     void* workspace = nullptr;    // non-null: N*bs elements of intermediate storage; `out` then holds N*bs only
     bool main_row = false;        // run the plan's own row whatever the batch (pieces of a larger batch)
+    void* pair_ws = nullptr;      // set for the plan of a fused pair: the turbofft_plan::PairWs to run it with
 };
 
 static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long long bs, void* stream, const exec_opts& o);
@@ -943,22 +1050,44 @@ static bool ensure_part_slots(turbofft_plan* p, void* stream) {
     return true;
 }
 
-// The row a batch of `bs` transforms runs: the small-batch row (plain built-in plans, bs up to its cap) or the plan's own
+// The row a batch of `bs` transforms runs: the small-batch row (plain built-in plans, bs up to its cap), the fused
+// pair (batches that give every team a piece) or the plan's own
 static const turbofft_plan* row_for_batch(const turbofft_plan* p, long long bs) {
-    return (p->small && p->small_enabled && bs >= 1 && bs <= p->small_max_bs) ? p->small : p;
+    if (p->small && p->small_enabled && bs >= 1 && bs <= p->small_max_bs) return p->small;
+    if (p->pair && p->pair_enabled && (bs + p->pair->pair_per_piece - 1) / p->pair->pair_per_piece >= 8ll * p->pair->pair_teams_per_xcd) return p->pair;
+    return p;
 }
 
 int turbofft_plan_launches_for_batch(const turbofft_plan_t* p, long long bs) {
     if (!p || bs < 0) return fail(TURBOFFT_EINVAL, "bad argument");
-    return row_for_batch(p, bs)->launches;
+    const turbofft_plan* q = row_for_batch(p, bs);
+    return q->pk ? 1 : q->launches;
 }
 
 const char* turbofft_plan_kernel_name_for_batch(const turbofft_plan_t* p, int launch, long long bs) {
     if (!p || bs < 0) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
     const turbofft_plan* q = row_for_batch(p, bs);
-    if (launch < 0 || launch >= q->launches) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
+    if (launch < 0 || launch >= (q->pk ? 1 : q->launches)) { fail(TURBOFFT_EINVAL, "bad argument"); return nullptr; }
+    if (q->pk) return q->pk->name;
     const tfft_kernel_entry* k = launch_kernel(q, launch, false);
     return k ? k->name : nullptr;
+}
+
+int turbofft_plan_set_fused(turbofft_plan_t* p, int enable) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    if (enable && !p->pair) return fail(TURBOFFT_ENOPLAN, "the plan holds no fused kernel (none for this size, or created without TURBOFFT_FUSED=1)");
+    p->pair_enabled = enable != 0;
+    return TURBOFFT_OK;
+}
+
+int turbofft_plan_fused_info(const turbofft_plan_t* p, int* team_blocks, int* transforms_per_piece, int* teams_per_xcd, int* grid_blocks) {
+    if (!p) return fail(TURBOFFT_EINVAL, "null plan");
+    const turbofft_plan* q = p->pair;
+    if (team_blocks) *team_blocks = q ? q->pair_team : 0;
+    if (transforms_per_piece) *transforms_per_piece = q ? q->pair_per_piece : 0;
+    if (teams_per_xcd) *teams_per_xcd = q ? q->pair_teams_per_xcd : 0;
+    if (grid_blocks) *grid_blocks = q ? q->pair_grid : 0;
+    return (q && p->pair_enabled) ? 1 : 0;
 }
 
 static bool ranges_overlap(const void* a, size_t an, const void* b, size_t bn) {
@@ -1013,6 +1142,36 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         return exec_impl(p->small, in_d, out_d, bs, stream, so);
         }
     }
+    if (p->pair && p->pair_enabled && !inverse && !o.main_row && !o.ev &&
+        (bs + p->pair->pair_per_piece - 1) / p->pair->pair_per_piece >= 8ll * p->pair->pair_teams_per_xcd) {
+        // both launches as one kernel, where every team gets at least one piece: the slots and control block of this
+        // stream (a stream without a set gets one now, unless it is being captured or the plan keeps kMaxPairWs
+        // already: then the two launches run)
+        turbofft_plan::PairWs* w = nullptr;
+        {
+            std::lock_guard<std::mutex> lk(p->pair_mu);
+            for (auto& e : p->pair_ws) if (e.assigned && e.stream == stream) { w = &e; break; }
+            if (!w) for (auto& e : p->pair_ws) if (!e.assigned) { e.assigned = true; e.stream = stream; w = &e; break; }
+            // (a caller that brought its own workspace may be one that cannot allocate: no new set for it)
+            if (!w && !o.workspace && p->pair_ws.size() < kMaxPairWs && !stream_is_capturing(stream) && pair_add_ws(p, p->pair, stream, true)) w = &p->pair_ws.back();
+        }
+        if (w) {
+            if (*(volatile unsigned*)w->err_host) {
+                // an earlier execution on this stream gave up waiting (its blocks were not all resident in time):
+                // what it left in `out` is incomplete.  The plan goes back to its two launches.
+                *(volatile unsigned*)w->err_host = 0u;
+                p->pair_enabled = false;
+                return fail(TURBOFFT_EHIP, "an earlier execution of the fused kernel of this plan ran out of time waiting for its blocks to be "
+                            "resident together; its output is incomplete.  The plan runs its two launches from now on");
+            }
+            if (ranges_overlap(in_d, data_bytes, out, data_bytes))
+                return fail(TURBOFFT_EINVAL, "in [%p, +%zu) overlaps out [%p, ...): the transform is out of place", in_d, data_bytes, (void*)out);
+            p->last_stream.store(stream, std::memory_order_release);
+            exec_opts po = o;
+            po.pair_ws = w;
+            return exec_impl(p->pair, in_d, out_d, bs, stream, po);
+        }
+    }
     const Row& r = p->row;
     char* work = o.workspace ? (char*)o.workspace : out + data_bytes;
     // The transform is out of place: the kernels read `in` while they write `out` (and a
@@ -1031,6 +1190,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
     else if (p->launches == 2) { src[0] = in_d; dst[0] = work; src[1] = work; dst[1] = out; }
     else { src[0] = in_d; dst[0] = out; src[1] = out; dst[1] = work; src[2] = work; dst[2] = out; }
     p->last_stream.store(stream, std::memory_order_release);
+    tfft_kargs pair_args[2];
     for (int i = 0; i < p->launches; ++i) {
         const tfft_kernel_entry* k = launch_kernel(p, i, inverse);
         tfft_kargs a;
@@ -1078,6 +1238,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             a.ft.err_smoothing = p->err_smoothing;
             a.ft.err_threshold = p->err_threshold;
         }
+        if (o.pair_ws) { pair_args[i] = a; continue; }     // the fused kernel takes both launches' arguments
         long long grid = (a.ntiles + a.thread_bs - 1) / a.thread_bs;
         if (grid < 1) continue;
         long long fix_grid = 0;
@@ -1114,6 +1275,46 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
                                     (hipStream_t)stream));
         }
         if (o.sync_each) HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    }
+    if (o.pair_ws) {
+        const turbofft_plan::PairWs* w = (const turbofft_plan::PairWs*)o.pair_ws;
+        tfft_fuse_args f;
+        memset(&f, 0, sizeof f);
+        f.slots = w->slots;
+        f.ctl = w->ctl;
+        f.err_host = w->err_host;
+        f.piece_elems = (long long)p->pair_per_piece << p->logN;
+        f.npieces = (bs + p->pair_per_piece - 1) / p->pair_per_piece;
+        f.tiles_a = p->pair_per_piece * ((1 << r.logNi(1)) / r.BS(0));
+        f.tiles_b = p->pair_per_piece * ((1 << r.logNi(0)) / r.BS(1));
+        f.team = p->pair_team;
+        f.teams_per_xcd = p->pair_teams_per_xcd;
+        f.limit_ms = p->pair_limit_ms;
+        if (getenv("TURBOFFT_FUSED_PROF")) {
+            // diagnostic (kernels built with TFFT_PAIR_PROFILE set): time per part of a round, printed per execution
+            static unsigned long long* prof = nullptr;
+            if (!prof) { if (hipMalloc((void**)&prof, 8 * sizeof(unsigned long long) * 65536) != hipSuccess) prof = nullptr; }
+            f.prof = prof;
+        }
+        if (f.npieces > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "too many pieces for the fused kernel");
+        const void* in_arg = in_d;
+        void* out_arg = out;
+        const void* tw_arg = p->tw;
+        void* args[6] = {(void*)&in_arg, (void*)&out_arg, (void*)&tw_arg, (void*)&pair_args[0], (void*)&pair_args[1], (void*)&f};
+        HIP_TRY(hipLaunchKernel(p->pk->func, dim3((unsigned)p->pair_grid), dim3((unsigned)p->pk->threads), args, (size_t)p->pk->lds_bytes,
+                                (hipStream_t)stream));
+        if (o.sync_each) HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+        if (f.prof && getenv("TURBOFFT_FUSED_PROF") && atoi(getenv("TURBOFFT_FUSED_PROF")) == 2) {
+            HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+            std::vector<unsigned long long> h((size_t)8 * p->pair_grid);
+            HIP_TRY(hipMemcpy(h.data(), f.prof, h.size() * 8, hipMemcpyDeviceToHost));
+            double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int b = 0; b < p->pair_grid; ++b) for (int k = 0; k < 8; ++k) t[k] += (double)h[8 * b + k];
+            const double rounds = t[4] > 0 ? t[4] : 1;
+            fprintf(stderr, "fused %s: per round, us: column launch %.2f, meeting %.2f, row launch: first phase %.2f, fetch ahead %.2f, rest %.2f, slot wait %.2f (%.1f rounds per block)\n",
+                    p->pk->name, t[0] / rounds / 100, t[1] / rounds / 100, t[5] / rounds / 100, t[6] / rounds / 100, t[2] / rounds / 100, t[3] / rounds / 100, t[4] / p->pair_grid);
+        }
+        return TURBOFFT_OK;
     }
     if (o.ev) HIP_TRY(hipEventRecord(o.ev[p->launches], (hipStream_t)stream));
     return TURBOFFT_OK;

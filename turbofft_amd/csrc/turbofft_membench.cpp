@@ -5,6 +5,7 @@
 // Measurement only: nothing here is used by turbofft_exec.  No counterpart in the reference, which
 // quotes its bandwidth against the data sheet (readme.md).
 #include <hip/hip_runtime.h>
+#include <cstring>
 
 #include "../../include/turbofft.h"
 
@@ -102,11 +103,11 @@ __global__ __launch_bounds__(256) void tfft_mb_strided(const V* __restrict__ in,
 
 // ---- two passes through a ring that stays in the XCD's L2 (the question a fused pass pair of a
 // two-launch plan would have to answer first) ----
-// Synthetic: in -> ring -> out as ONE persistent kernel.  The data is cut into "transforms" of 512 KiB;
+// Synthetic: in -> ring -> out as ONE persistent kernel (`lag`: how many groups the second pass runs behind the first in ticket order).  The data is cut into "transforms" of 512 KiB;
 // each of the 8 XCDs (a block reads its XCD from the hardware register) owns every eighth transform and a
 // ring of R slots of G transforms that is reused for every group, so the intermediate is only ever written
 // to addresses that are still in that XCD's L2.  Items are handed out per XCD in ticket order
-//   P1(g0) | P1(g1) P2(g0) | P1(g2) P2(g1) | ...
+//   P1(g0) | P1(g1) P2(g0) | P1(g2) P2(g1) | ...          (lag 1; with lag K: P1(g0) ... P1(gK-1) | P1(gK) P2(g0) | ...)
 // (P1: 32 KiB of a transform in -> slot, 16 per transform; P2: 64 KiB slot -> out, 8 per transform).  A P2
 // item needs every P1 item of its group (as a row pass needs every column tile), a P1 item of group g
 // needs slot g % R drained by P2(g - R).  Every wait is for items with lower tickets, which running blocks
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(256) void tfft_mb_strided(const V* __restrict__ in,
 constexpr long long kFusedTransform = 512 << 10;
 constexpr int kFusedP1 = 32 << 10, kFusedP2 = 64 << 10, kFusedMaxGroups = 2048;
 struct FusedQueue { unsigned next; unsigned pad0[31]; unsigned done1[kFusedMaxGroups]; unsigned done2[kFusedMaxGroups]; };
-struct FusedCtl { unsigned err, waits, spins, pad[29]; unsigned xcc_blocks[32]; FusedQueue q[8]; };
+struct FusedCtl { unsigned err, pad0[31]; unsigned waits, spins, pad1[30]; unsigned xcc_blocks[32]; FusedQueue q[8]; };   // the flag every block reads has a line of its own
 
 __global__ void tfft_mb_fused_clear(FusedCtl* c) {
     const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -131,23 +132,27 @@ __device__ __forceinline__ void fused_copy_item(const char* src, char* dst) {
     for (int e = 0; e < U; ++e) __builtin_amdgcn_raw_buffer_store_b128(r[e], mb_rsrc(dst), (threadIdx.x + e * 256) * 16u, 0, SAUX);
 }
 
-// thread 0 waits until *p >= k; false after the time limit or when another block gave up
-__device__ __forceinline__ bool fused_wait(unsigned* p, unsigned k, FusedCtl* c, long long t_limit) {
+// thread 0 waits until *p >= k; false after the time limit or when another block gave up.  The statistics stay in the
+// caller's registers until the block ends and the give-up flag is read on every eighth poll: counters that every
+// waiting block updates in one line serialise the waits of the whole grid.
+__device__ __forceinline__ bool fused_wait(unsigned* p, unsigned k, FusedCtl* c, long long t_limit, unsigned& waits, unsigned& spins_total) {
     unsigned spins = 0;
     for (;;) {
         if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= k) {
-            if (spins) { atomicAdd(&c->waits, 1u); atomicAdd(&c->spins, spins); }
+            if (spins) { ++waits; spins_total += spins; }
             return true;
         }
-        if (__hip_atomic_load(&c->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
-        if ((long long)wall_clock64() > t_limit) { atomicExch(&c->err, 1u); return false; }
-        __builtin_amdgcn_s_sleep(8);
+        if ((spins & 7u) == 7u) {
+            if (__hip_atomic_load(&c->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+            if ((long long)wall_clock64() > t_limit) { atomicExch(&c->err, 1u); return false; }
+        }
+        __builtin_amdgcn_s_sleep(2);
         ++spins;
     }
 }
 
 __global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in, char* __restrict__ scratch, char* __restrict__ out, FusedCtl* c,
-                                                    int ntrans_per_xcd, int G, int R, int limit_ms) {
+                                                    int ntrans_per_xcd, int G, int R, int limit_ms, int lag) {
     __shared__ unsigned s_t;
     __shared__ int s_ok;
     const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;     // XCC_ID[3:0] of the hardware register
@@ -158,6 +163,7 @@ __global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in
     const unsigned n1 = (unsigned)(kFusedTransform / kFusedP1 * G), n2 = (unsigned)(kFusedTransform / kFusedP2 * G);
     const unsigned total = (unsigned)ngroups * (n1 + n2);
     char* ring = scratch + (size_t)xcc * R * G * kFusedTransform;
+    unsigned waits = 0, spins = 0;
     for (;;) {
         if (threadIdx.x == 0) {
             unsigned t = atomicAdd(&q->next, 1u);
@@ -168,17 +174,18 @@ __global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in
         const unsigned t = (unsigned)__builtin_amdgcn_readfirstlane((int)s_t);
         __syncthreads();
         if (t >= total) break;
+        // ticket order with the second pass `lag` groups behind the first: segment s holds P1(s) (s < ngroups) then P2(s - lag) (s >= lag)
         bool is1; unsigned g, i;
-        if (t < n1) { is1 = true; g = 0; i = t; }
-        else {
-            const unsigned u = t - n1, seg = u / (n1 + n2), r = u % (n1 + n2);
-            if (seg + 1 < (unsigned)ngroups) { if (r < n1) { is1 = true; g = seg + 1; i = r; } else { is1 = false; g = seg; i = r - n1; } }
-            else { is1 = false; g = (unsigned)ngroups - 1; i = r; }
-        }
+        const unsigned K = (unsigned)lag, head = K * n1, mid = ((unsigned)ngroups - K) * (n1 + n2);
+        if (t < head) { is1 = true; g = t / n1; i = t % n1; }
+        else if (t - head < mid) {
+            const unsigned u = t - head, seg = K + u / (n1 + n2), r = u % (n1 + n2);
+            if (r < n1) { is1 = true; g = seg; i = r; } else { is1 = false; g = seg - K; i = r - n1; }
+        } else { const unsigned u = t - head - mid; is1 = false; g = (unsigned)ngroups - K + u / n2; i = u % n2; }
         char* slot = ring + (size_t)(g % R) * G * kFusedTransform;
         if (is1) {
             if (g >= (unsigned)R) {
-                if (threadIdx.x == 0) s_ok = fused_wait(&q->done2[g - R], n2, c, t_limit) ? 1 : 0;
+                if (threadIdx.x == 0) s_ok = fused_wait(&q->done2[g - R], n2, c, t_limit, waits, spins) ? 1 : 0;
                 __syncthreads();
                 const int ok = s_ok;
                 __syncthreads();
@@ -191,7 +198,7 @@ __global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in
             __syncthreads();
             if (threadIdx.x == 0) atomicAdd(&q->done1[g], 1u);
         } else {
-            if (threadIdx.x == 0) s_ok = fused_wait(&q->done1[g], n1, c, t_limit) ? 1 : 0;
+            if (threadIdx.x == 0) s_ok = fused_wait(&q->done1[g], n1, c, t_limit, waits, spins) ? 1 : 0;
             __syncthreads();
             const int ok = s_ok;
             __syncthreads();
@@ -199,11 +206,142 @@ __global__ __launch_bounds__(256) void tfft_mb_fused(const char* __restrict__ in
             const unsigned per = (unsigned)(kFusedTransform / kFusedP2), k = i / per, j = i % per;
             const size_t T = (size_t)(g * G + k) * 8 + xcc;
             // agent-scope loads of the ring: never served from this CU's L1, which may hold the slot's previous contents
-            fused_copy_item<kFusedP2 / 4096, 16, 2>(slot + (size_t)k * kFusedTransform + (size_t)j * kFusedP2, out + T * kFusedTransform + (size_t)j * kFusedP2);
-            __builtin_amdgcn_s_waitcnt(0x0F70);       // the slot's loads have returned before it is handed back
-            __syncthreads();
+            constexpr int U2 = kFusedP2 / 4096;
+            const char* from = slot + (size_t)k * kFusedTransform + (size_t)j * kFusedP2;
+            char* to = out + T * kFusedTransform + (size_t)j * kFusedP2;
+            u4 r[U2];
+#pragma unroll
+            for (int e = 0; e < U2; ++e) r[e] = __builtin_amdgcn_raw_buffer_load_b128(mb_rsrc(from), (threadIdx.x + e * 256) * 16u, 0, 16);
+            __builtin_amdgcn_s_waitcnt(0x0F70);       // the slot's loads have returned: it is handed back before the stores to
+            __syncthreads();                          // memory are issued, whose acknowledgement nobody waits for here
             if (threadIdx.x == 0) atomicAdd(&q->done2[g], 1u);
+#pragma unroll
+            for (int e = 0; e < U2; ++e) __builtin_amdgcn_raw_buffer_store_b128(r[e], mb_rsrc(to), (threadIdx.x + e * 256) * 16u, 0, 2);
         }
+    }
+    if (threadIdx.x == 0 && waits) { atomicAdd(&c->waits, waits); atomicAdd(&c->spins, spins); }
+}
+
+// ---- the same question with teams: T blocks of one XCD share one 512 KiB piece at a time ----
+// Every team owns ONE slot, reused for every piece it handles, so an XCD's slots (teams x 512 KiB) are all the
+// intermediate there is.  Per piece: every member copies its 1/T of the piece in -> slot, the team meets at a
+// barrier (a counter per team, agent-scope atomics, bounded polling), every member copies another 1/T of the slot
+// (2 KiB from each member's part, as a row tile takes a strip of every column tile) slot -> out, and the team meets
+// again before the slot is overwritten -- that second wait is taken after the next piece's loads have been issued.
+// Needs every block of the grid resident at once (the grid is sized from the occupancy query) and the blocks dealt
+// evenly to the XCDs; a member that never shows up ends in the time limit and the error flag, not in a hang.
+struct TeamBar { unsigned a, pad0[31]; unsigned b, pad1[31]; };      // one line for each counter
+struct TeamCtl { unsigned err, pad0[31]; unsigned waits, polls, pad1[30]; unsigned arrive[32]; unsigned long long ticks[16]; TeamBar bar[8][64]; };
+
+__global__ void tfft_mb_team_clear(TeamCtl* c) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < sizeof(TeamCtl) / 4) ((unsigned*)c)[i] = 0;
+}
+
+// One thread's wait for a counter of its team.  The flag that ends every wait after a time-out sits in a line of its
+// own and is read on every eighth poll only, and the statistics stay in the caller's registers until the block ends:
+// a line that every waiting block reads and updates would serialise the waits of the whole grid.
+__device__ __forceinline__ bool team_wait(unsigned* p, unsigned k, TeamCtl* c, long long t_limit, unsigned& waits, unsigned& polls_total) {
+    unsigned polls = 0;
+    for (;;) {
+        if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= k) {
+            if (polls) { ++waits; polls_total += polls; }
+            return true;
+        }
+        if ((polls & 7u) == 7u) {
+            if (__hip_atomic_load(&c->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+            if ((long long)wall_clock64() > t_limit) { atomicExch(&c->err, 1u); return false; }
+        }
+        __builtin_amdgcn_s_sleep(2);
+        ++polls;
+    }
+}
+
+// T: blocks per team; PIECE: bytes a team moves per round (one slot); every member moves PIECE / T per pass
+// POL: cache policy of the accesses to memory, loads of `in` in bits 0-1 and stores to `out` in bits 2-3:
+// 0 nt, 1 nt + sc0, 2 nt + sc1, 3 nt + sc0 + sc1.  The slot is written with the default policy; how it is read is bits 4-5:
+// 0 sc1 loads, 1 sc0 loads, 2 nt loads, 3 default loads behind an invalidation of the CU's vector L1 (buffer_inv sc1)
+template <int T, int PIECE, int POL = 0>
+__global__ __launch_bounds__(256) void tfft_mb_team(const char* __restrict__ in, char* __restrict__ scratch, char* __restrict__ out, TeamCtl* c,
+                                                   int ntrans, int limit_ms) {
+    constexpr int SHARE = PIECE / T, U = SHARE / 4096;
+    constexpr int kAux[4] = {2, 3, 18, 19};
+    constexpr int LAUX = kAux[POL & 3], SAUX = kAux[(POL >> 2) & 3];
+    constexpr int kSlotAux[4] = {16, 1, 2, 0};
+    constexpr int RAUX = kSlotAux[(POL >> 4) & 3];
+    static_assert(U >= 1 && U <= 32 && SHARE / T >= 16, "a share fits the registers of a block");      // bytes per member and pass; 16-byte accesses per thread
+    __shared__ unsigned s_idx;
+    __shared__ int s_ok;
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;
+    const long long t_limit = (long long)wall_clock64() + (long long)limit_ms * 100000ll;
+    if (threadIdx.x == 0) s_idx = atomicAdd(&c->arrive[xcc], 1u);
+    __syncthreads();
+    const unsigned idx = (unsigned)__builtin_amdgcn_readfirstlane((int)s_idx);
+    const unsigned nteams = (gridDim.x / 8u) / (unsigned)T;
+    const unsigned team = idx / (unsigned)T, member = idx % (unsigned)T;
+    if (team >= nteams) return;                                   // blocks beyond whole teams have nothing to do
+    TeamBar* bar = &c->bar[xcc][team];
+    char* slot = scratch + ((size_t)xcc * nteams + team) * (size_t)PIECE;
+    u4 r[U];
+    unsigned round = 0, waits = 0, polls = 0;
+    // time per part of a round as thread 0 sees it (100 MHz ticks): [0] until the piece's loads have returned, [1] the wait for
+    // the slot, [2] slot stores acknowledged, [3] the team barrier, [4] the slot's loads have returned, [5] the rest
+    long long tk[6] = {0, 0, 0, 0, 0, 0}, tl = (long long)wall_clock64();
+#define MB_TICK(k) { const long long now_ = (long long)wall_clock64(); tk[k] += now_ - tl; tl = now_; }
+    for (size_t t = xcc + 8 * (size_t)team; t < (size_t)ntrans; t += 8 * (size_t)nteams, ++round) {
+        // pass 1: this member's contiguous part of the piece
+        const char* src = in + t * (size_t)PIECE + (size_t)member * SHARE;
+#pragma unroll
+        for (int e = 0; e < U; ++e) r[e] = __builtin_amdgcn_raw_buffer_load_b128(mb_rsrc(src), (threadIdx.x + e * 256) * 16u, 0, LAUX);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        MB_TICK(0)
+        if (round) {                                               // the slot's previous contents have been read by every member
+            if (threadIdx.x == 0) s_ok = team_wait(&bar->b, (unsigned)T * round, c, t_limit, waits, polls) ? 1 : 0;
+            __syncthreads();
+            const int ok = s_ok;
+            __syncthreads();
+            if (!ok) return;
+        }
+        MB_TICK(1)
+        char* mine = slot + (size_t)member * SHARE;
+#pragma unroll
+        for (int e = 0; e < U; ++e) __builtin_amdgcn_raw_buffer_store_b128(r[e], mb_rsrc(mine), (threadIdx.x + e * 256) * 16u, 0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        MB_TICK(2)
+        __syncthreads();
+        if (threadIdx.x == 0) { atomicAdd(&bar->a, 1u); s_ok = team_wait(&bar->a, (unsigned)T * (round + 1), c, t_limit, waits, polls) ? 1 : 0; }
+        __syncthreads();
+        const int ok1 = s_ok;
+        __syncthreads();
+        if (!ok1) return;
+        MB_TICK(3)
+        // pass 2: a strip of every member's part: piece j of this member's second-pass share is bytes
+        // [member * (SHARE / T), +SHARE / T) of member j's part
+        if constexpr (((POL >> 4) & 3) == 3) asm volatile("buffer_inv sc1" ::: "memory");   // nothing of the slot's last contents is left in this CU's L1
+        constexpr int STRIP = SHARE / T;                           // bytes taken from each part
+        constexpr int PER = STRIP / 16;                            // 16-byte accesses per strip
+#pragma unroll
+        for (int e = 0; e < U; ++e) {
+            const unsigned q = threadIdx.x + e * 256, j = q / PER, w = q % PER;
+            r[e] = __builtin_amdgcn_raw_buffer_load_b128(mb_rsrc(slot), j * (unsigned)SHARE + member * (unsigned)STRIP + w * 16u, 0, RAUX);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);                        // the slot's loads have returned: hand the slot back before the stores
+        MB_TICK(4)
+        __syncthreads();                                           // to memory are issued, whose acknowledgement nobody has to wait for here
+        if (threadIdx.x == 0) atomicAdd(&bar->b, 1u);
+        char* dst = out + t * (size_t)PIECE;
+#pragma unroll
+        for (int e = 0; e < U; ++e) {
+            const unsigned q = threadIdx.x + e * 256, j = q / PER, w = q % PER;
+            __builtin_amdgcn_raw_buffer_store_b128(r[e], mb_rsrc(dst), j * (unsigned)SHARE + member * (unsigned)STRIP + w * 16u, 0, SAUX);
+        }
+        MB_TICK(5)
+    }
+#undef MB_TICK
+    if (threadIdx.x == 0) {
+        if (waits) { atomicAdd(&c->waits, waits); atomicAdd(&c->polls, polls); }
+        for (int k = 0; k < 6; ++k) atomicAdd(&c->ticks[k], (unsigned long long)tk[k]);
+        atomicAdd(&c->ticks[6], (unsigned long long)round);
     }
 }
 
@@ -254,15 +392,15 @@ extern "C" int turbofft_membench_strided(int write, int lane_bytes, int run_byte
     return mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
 }
 
-extern "C" int turbofft_membench_fused(int group, int ring_slots, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+extern "C" int turbofft_membench_fused(int group, int ring_slots, int lag, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
                                        void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
                                        unsigned stats[12]) {
     if (!src_d || !dst_d || !scratch_d || !ms_per_pass || !stats || reps < 1 || warmup < 0) { tfft_set_error("membench: bad argument"); return TURBOFFT_EINVAL; }
     const long long ntrans = (long long)(bytes / kFusedTransform), per_xcd = ntrans / 8;
-    // (R >= 2: P1 of group g waits for P2 of group g - R, which has to come earlier in ticket order)
-    if (bytes == 0 || bytes % (8 * kFusedTransform) || group < 1 || ring_slots < 2 || ring_slots > 8 || per_xcd % group || per_xcd / group > kFusedMaxGroups ||
+    // (R > lag: P1 of group g waits for P2 of group g - R, which has to come earlier in ticket order: segment g - R + lag < g)
+    if (bytes == 0 || bytes % (8 * kFusedTransform) || group < 1 || lag < 1 || ring_slots <= lag || ring_slots > 16 || per_xcd % group || per_xcd / group > kFusedMaxGroups || per_xcd / group <= lag ||
         blocks_per_cu < 1 || blocks_per_cu > 8 || limit_ms < 1 || limit_ms > 1000 || (unsigned long long)8 * ring_slots * group * kFusedTransform > scratch_bytes) {
-        tfft_set_error("membench: fused copy needs bytes a multiple of 4 MiB, 2..8 ring slots of `group` 512 KiB transforms per XCD inside `scratch`, "
+        tfft_set_error("membench: fused copy needs bytes a multiple of 4 MiB, lag >= 1, lag+1..16 ring slots of `group` 512 KiB transforms per XCD inside `scratch`, "
                        "at most %d groups per XCD, 1..8 blocks per CU and a time limit of 1..1000 ms", kFusedMaxGroups);
         return TURBOFFT_EINVAL;
     }
@@ -280,15 +418,88 @@ extern "C" int turbofft_membench_fused(int group, int ring_slots, int blocks_per
     const unsigned grid = (unsigned)(cus * blocks_per_cu);
     auto launch = [&]() {
         hipLaunchKernelGGL(tfft_mb_fused_clear, dim3((unsigned)((sizeof(FusedCtl) / 4 + 255) / 256)), dim3(256), 0, st, ctl);
-        hipLaunchKernelGGL(tfft_mb_fused, dim3(grid), dim3(256), 0, st, (const char*)src_d, (char*)scratch_d, (char*)dst_d, ctl, (int)per_xcd, group, ring_slots, limit_ms);
+        hipLaunchKernelGGL(tfft_mb_fused, dim3(grid), dim3(256), 0, st, (const char*)src_d, (char*)scratch_d, (char*)dst_d, ctl, (int)per_xcd, group, ring_slots, limit_ms, lag);
     };
     int rc = mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
-    unsigned head[64];
+    unsigned head[96];
     if (rc == TURBOFFT_OK && hipMemcpy(head, ctl, sizeof head, hipMemcpyDeviceToHost) != hipSuccess) { (void)hipGetLastError(); tfft_set_error("membench: reading the control block failed"); rc = TURBOFFT_EHIP; }
     (void)hipFree(ctl);
     if (rc) return rc;
-    stats[0] = head[0]; stats[1] = head[1]; stats[2] = head[2]; stats[3] = grid;      // error flag, waits, polls, blocks
-    for (int x = 0; x < 8; ++x) stats[4 + x] = head[32 + x];                          // blocks that ran on each XCD
+    stats[0] = head[0]; stats[1] = head[32]; stats[2] = head[33]; stats[3] = grid;    // error flag, waits, polls, blocks
+    for (int x = 0; x < 8; ++x) stats[4 + x] = head[64 + x];                          // blocks that ran on each XCD
+    return TURBOFFT_OK;
+}
+
+template <int T, int PIECE>
+static const void* mb_team_fn() {
+    if constexpr (PIECE / T >= 4096 && PIECE / T <= 131072 && PIECE / T / T >= 16) return (const void*)tfft_mb_team<T, PIECE>;
+    else return nullptr;
+}
+template <int POL>
+static const void* mb_team_pol(int policy) {      // the other cache policies: teams of 8 with pieces of 512 KiB only
+    if constexpr (POL > 63) return nullptr;
+    else return policy == POL ? (const void*)tfft_mb_team<8, 512 << 10, POL> : mb_team_pol<POL + 1>(policy);
+}
+template <int PIECE>
+static const void* mb_team_fn_t(int team_blocks) {
+    switch (team_blocks) {
+        case 4: return mb_team_fn<4, PIECE>();
+        case 8: return mb_team_fn<8, PIECE>();
+        case 16: return mb_team_fn<16, PIECE>();
+        case 32: return mb_team_fn<32, PIECE>();
+        default: return nullptr;
+    }
+}
+
+extern "C" int turbofft_membench_team(int team_blocks, int piece_kib, int policy, int blocks_per_cu, const void* src_d, void* scratch_d, size_t scratch_bytes,
+                                      void* dst_d, size_t bytes, int limit_ms, int warmup, int reps, void* stream, float* ms_per_pass,
+                                      unsigned stats[12]) {
+    if (!src_d || !dst_d || !scratch_d || !ms_per_pass || !stats || reps < 1 || warmup < 0) { tfft_set_error("membench: bad argument"); return TURBOFFT_EINVAL; }
+    const void* fn = nullptr;
+    fn = piece_kib == 128 ? mb_team_fn_t<128 << 10>(team_blocks) : piece_kib == 256 ? mb_team_fn_t<256 << 10>(team_blocks)
+                   : piece_kib == 512 ? mb_team_fn_t<512 << 10>(team_blocks) : piece_kib == 1024 ? mb_team_fn_t<1024 << 10>(team_blocks) : nullptr;
+    if (policy) fn = (team_blocks == 8 && piece_kib == 512) ? mb_team_pol<1>(policy) : nullptr;
+    const size_t piece = (size_t)piece_kib << 10;
+    if (!fn || bytes == 0 || bytes % (8 * piece) || blocks_per_cu < 1 || blocks_per_cu > 8 || limit_ms < 1 || limit_ms > 1000) {
+        tfft_set_error("membench: team copy needs teams of 4, 8, 16 or 32 blocks, pieces of 128, 256, 512 or 1024 KiB with 4..128 KiB per member, "
+                       "bytes a multiple of 8 pieces, 1..8 blocks per CU and a time limit of 1..1000 ms");
+        return TURBOFFT_EINVAL;
+    }
+    int dev = 0, cus = 0, occ = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, 256, 0) != hipSuccess || occ < 1) {
+        (void)hipGetLastError();
+        tfft_set_error("membench: cannot size the persistent grid");
+        return TURBOFFT_EHIP;
+    }
+    if (blocks_per_cu > occ) blocks_per_cu = occ;           // every block has to be resident: its team waits for it
+    const unsigned grid = (unsigned)(cus * blocks_per_cu), nteams = (grid / 8) / (unsigned)team_blocks;
+    if (nteams < 1 || nteams > 64 || (unsigned long long)8 * nteams * piece > scratch_bytes) {
+        tfft_set_error("membench: %u teams per XCD need 1..64 slots of %d KiB per XCD inside `scratch`", nteams, piece_kib);
+        return TURBOFFT_EINVAL;
+    }
+    TeamCtl* ctl = nullptr;
+    if (hipMalloc((void**)&ctl, sizeof(TeamCtl)) != hipSuccess) { (void)hipGetLastError(); tfft_set_error("membench: hipMalloc failed"); return TURBOFFT_ENOMEM; }
+    hipStream_t st = (hipStream_t)stream;
+    const int ntrans = (int)(bytes / piece);
+    auto launch = [&]() {
+        hipLaunchKernelGGL(tfft_mb_team_clear, dim3((unsigned)((sizeof(TeamCtl) / 4 + 255) / 256)), dim3(256), 0, st, ctl);
+        const char* in_a = (const char*)src_d; char* sc_a = (char*)scratch_d; char* out_a = (char*)dst_d; int nt = ntrans, lm = limit_ms;
+        void* args[6] = {&in_a, &sc_a, &out_a, &ctl, &nt, &lm};
+        (void)hipLaunchKernel(fn, dim3(grid), dim3(256), args, 0, st);
+    };
+    int rc = mb_time(launch, warmup, reps, st, ms_per_pass, "membench");
+    unsigned head[128];
+    if (rc == TURBOFFT_OK && hipMemcpy(head, ctl, sizeof head, hipMemcpyDeviceToHost) != hipSuccess) { (void)hipGetLastError(); tfft_set_error("membench: reading the control block failed"); rc = TURBOFFT_EHIP; }
+    (void)hipFree(ctl);
+    if (rc) return rc;
+    stats[0] = head[0]; stats[1] = head[32]; stats[2] = head[33]; stats[3] = grid;
+    // [4..9]: mean time per round of each part, in ticks of 10 ns; [10]: rounds per block; [11]: unused
+    unsigned long long tk[7];
+    memcpy(tk, head + 96, sizeof tk);
+    for (int k = 0; k < 6; ++k) stats[4 + k] = tk[6] ? (unsigned)(tk[k] / tk[6]) : 0u;
+    stats[10] = (unsigned)(tk[6] / (grid ? grid : 1));
+    stats[11] = 0;
     return TURBOFFT_OK;
 }
 
