@@ -1022,6 +1022,9 @@ class KernelEmitter:
                     if self.role == "A" and self.prefetched:
                         c.ind -= 1
                         c("}")
+                    if self.role == "B" and os.environ.get("TFFT_PAIR_PROFILE"):
+                        c("TFFT_WAIT_VMEM();")
+                        c("if (f.prof) { const long long now_ = (long long)wall_clock64(); pt[7] += now_ - pt_last; pt_last = now_; }")
                     if sp.dc:
                         c.ind -= 1
                         c("} else {")

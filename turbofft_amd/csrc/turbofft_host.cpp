@@ -1311,8 +1311,8 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
             double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             for (int b = 0; b < p->pair_grid; ++b) for (int k = 0; k < 8; ++k) t[k] += (double)h[8 * b + k];
             const double rounds = t[4] > 0 ? t[4] : 1;
-            fprintf(stderr, "fused %s: per round, us: column launch %.2f, meeting %.2f, row launch: first phase %.2f, fetch ahead %.2f, rest %.2f, slot wait %.2f (%.1f rounds per block)\n",
-                    p->pk->name, t[0] / rounds / 100, t[1] / rounds / 100, t[5] / rounds / 100, t[6] / rounds / 100, t[2] / rounds / 100, t[3] / rounds / 100, t[4] / p->pair_grid);
+            fprintf(stderr, "fused %s: per round, us: column launch %.2f, meeting %.2f, row launch: slot loads %.2f, first phase %.2f, fetch ahead %.2f, rest %.2f, slot wait %.2f (%.1f rounds per block)\n",
+                    p->pk->name, t[0] / rounds / 100, t[1] / rounds / 100, t[7] / rounds / 100, t[5] / rounds / 100, t[6] / rounds / 100, t[2] / rounds / 100, t[3] / rounds / 100, t[4] / p->pair_grid);
         }
         return TURBOFFT_OK;
     }
