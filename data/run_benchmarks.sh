@@ -25,6 +25,8 @@ for dt in 0 1; do
     run "$out/benchmark_TurboFFT_ft_${gpu}_$p.csv"  "turboFFT," --if_bench 2  --thread_bs 32 --datatype $dt --if_ft 1 --if_err 0
     run "$out/benchmark_TurboFFT_err_${gpu}_$p.csv" "turboFFT," --if_bench 2  --thread_bs 32 --datatype $dt --if_ft 1 --if_err 1
     run "$out/benchmark_hipFFT_${gpu}_$p.csv"       "hipFFT,"   --if_bench 12 --datatype $dt
+    # plans that hold the fused kernel of their two launches (fp32 2^16, fp64 2^15 and 2^16; the other sizes run as above)
+    TURBOFFT_FUSED=1 run "$out/benchmark_TurboFFT_fused_${gpu}_$p.csv" "turboFFT," --if_bench 2 --thread_bs 1 --datatype $dt --if_ft 0 --if_err 0
     for t in 1 2 4 8 16 32; do
         run "$out/ft/ft_scheme_threadblock_bs=${t}_${gpu}_$p.csv" "turboFFT," --if_bench 1 --thread_bs $t --datatype $dt --if_ft 1 --if_err 1
     done
