@@ -103,7 +103,8 @@ typedef struct tfft_fuse_args {
     int tiles_a, tiles_b;         /* tiles of the column launch and of the row launch per piece        */
     int team;                     /* blocks per team                                                  */
     int teams_per_xcd;
-    int limit_ms;                 /* longest time a block waits for other blocks                      */
+    int limit_ms;                 /* longest time a block waits for other blocks; negative: every block gives
+                                     up as it starts (sets word 0 and err_host, does nothing else)      */
     unsigned long long* prof;     /* diagnostic builds of the kernels only (else null): 8 words per block, ticks of the
                                      100 MHz counter spent in [0] the column launch, [1] the meeting, [2] the row launch,
                                      [3] the wait for the slot to be free, [4] rounds                                 */

@@ -956,3 +956,29 @@ def test_fused_pair_on_several_streams_and_in_a_graph(monkeypatch):
         torch.cuda.synchronize()
         assert torch.equal(out[: bs << logN].view(bs, -1), eager)
     plan.close()
+
+
+def test_fused_pair_that_gives_up_is_reported_and_replaced(monkeypatch):
+    # every wait of the fused kernel is bounded; with no time at all (a negative limit, set by the host) every block gives
+    # up as it starts and leaves.  The execution after that one reports it, and the plan runs its two launches from then on
+    torch = _torch()
+    monkeypatch.setenv("TURBOFFT_FUSED", "1")
+    monkeypatch.setenv("TURBOFFT_FUSED_LIMIT_MS", "-1")
+    dt, logN = "double2", 15
+    plan = turbofft_amd.TurboFFT(logN, dt)
+    info = plan.fused_info()
+    assert info is not None
+    bs = 8 * info["teams_per_xcd"] + 1
+    x = torch.from_numpy(make(bs, 1 << logN, dt, 4)).cuda()
+    out = torch.zeros(plan.out_elems(bs), dtype=x.dtype, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    plan.exec(x.data_ptr(), out.data_ptr(), bs, st)                 # launches; the kernel writes nothing
+    torch.cuda.synchronize()
+    assert not bool(out.any())
+    with pytest.raises(turbofft_amd.TurboFFTError, match="incomplete"):
+        plan.exec(x.data_ptr(), out.data_ptr(), bs, st)
+    assert plan.fused_info() is None and len(plan.kernel_names_for_batch(bs)) == 2
+    y = plan.fft(x)
+    torch.cuda.synchronize()
+    assert O.rel_l2(y.cpu().numpy(), O.fft_ref(x.cpu().numpy())) <= O.tolerance(dt, logN)
+    plan.close()

@@ -198,6 +198,14 @@ __device__ __forceinline__ bool tfft_team_join(const tfft_fuse_args& f, tfft_tea
     unsigned* base = f.ctl + 352 + 128 * (size_t)tm.slot;
     tm.a = base; tm.b = base + 32; tm.cur = (unsigned long long*)(base + 64);
     tm.t_limit = (long long)wall_clock64() + (long long)f.limit_ms * 100000ll;   // 100 MHz counter
+    if (f.limit_ms < 0) {
+        // no time at all (the host's way of exercising the give-up path): say so and take no part
+        if (threadIdx.x == 0) {
+            atomicExch(&f.ctl[0], 1u);
+            if (f.err_host) __hip_atomic_store(f.err_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        return false;
+    }
     return team < (unsigned)f.teams_per_xcd;
 }
 // The team's first piece, or -1 when there is none.  The leader waits until the team is complete -- or the queue

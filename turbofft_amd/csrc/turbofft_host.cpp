@@ -293,7 +293,8 @@ struct turbofft_plan {
     turbofft_plan* pair = nullptr;
     const tfft_pair_entry* pk = nullptr;
     int pair_team = 0, pair_per_piece = 0, pair_grid = 0, pair_teams_per_xcd = 0, pair_limit_ms = kPairLimitMs;
-    struct PairWs { void* stream; bool assigned; void* slots; unsigned* ctl; unsigned* err_host; };
+    struct PairWs { void* stream; bool assigned; void* slots; unsigned* ctl; unsigned* err_host; unsigned long long* prof; };
+    bool pair_prof = false;           // TURBOFFT_FUSED_PROF=1 at plan creation: diagnostic builds of the kernel leave their timings per execution
     std::vector<PairWs> pair_ws;
     std::mutex pair_mu;
     bool pair_enabled = true;
@@ -363,6 +364,7 @@ void turbofft_plan_destroy(turbofft_plan_t* p) {
         if (w.slots) (void)hipFree(w.slots);
         if (w.ctl) (void)hipFree(w.ctl);
         if (w.err_host) (void)hipHostFree(w.err_host);
+        if (w.prof) (void)hipFree(w.prof);
     }
     for (auto& w : p->small_ws) if (w.buf) (void)hipFree(w.buf);
     if (p->tw) (void)hipFree(p->tw);
@@ -435,18 +437,21 @@ static bool pair_add_ws(turbofft_plan* p, const turbofft_plan* q, void* stream, 
     const size_t nslots = (size_t)8 * q->pair_teams_per_xcd;
     const size_t slot_bytes = ((size_t)q->pair_per_piece << q->logN) * q->esize;
     const size_t ctl_bytes = sizeof(unsigned) * TFFT_FUSE_CTL_WORDS(nslots);
-    void *sl = nullptr, *ctl = nullptr, *eh = nullptr;
+    void *sl = nullptr, *ctl = nullptr, *eh = nullptr, *pf = nullptr;
+    const size_t prof_bytes = (size_t)8 * sizeof(unsigned long long) * (size_t)q->pair_grid;
     bool ok = hipMalloc(&sl, nslots * slot_bytes) == hipSuccess && hipMalloc(&ctl, ctl_bytes) == hipSuccess &&
-              hipHostMalloc(&eh, 64, hipHostMallocDefault) == hipSuccess && hipMemset(ctl, 0, ctl_bytes) == hipSuccess;
+              hipHostMalloc(&eh, 64, hipHostMallocDefault) == hipSuccess && hipMemset(ctl, 0, ctl_bytes) == hipSuccess &&
+              (!q->pair_prof || (hipMalloc(&pf, prof_bytes) == hipSuccess && hipMemset(pf, 0, prof_bytes) == hipSuccess));
     if (!ok) {
         (void)hipGetLastError();
         if (sl) (void)hipFree(sl);
         if (ctl) (void)hipFree(ctl);
         if (eh) (void)hipHostFree(eh);
+        if (pf) (void)hipFree(pf);
         return false;
     }
     *(volatile unsigned*)eh = 0u;
-    p->pair_ws.push_back({stream, assigned, sl, (unsigned*)ctl, (unsigned*)eh});
+    p->pair_ws.push_back({stream, assigned, sl, (unsigned*)ctl, (unsigned*)eh, (unsigned long long*)pf});
     return true;
 }
 
@@ -547,7 +552,9 @@ static int plan_build(turbofft_plan* p, const char* param_csv) {
             const int cus_per_xcd = prop.multiProcessorCount / 8, fit = cus_per_xcd * occ / q->pair_team;
             q->pair_teams_per_xcd = pr.teams() > 0 ? (pr.teams() < fit ? pr.teams() : fit) : cus_per_xcd / q->pair_team;
             q->pair_grid = 8 * q->pair_teams_per_xcd * q->pair_team;
-            if (const char* e = getenv("TURBOFFT_FUSED_LIMIT_MS")) if (atoi(e) > 0) q->pair_limit_ms = atoi(e);
+            // (a negative limit makes every block give up at once and leave: how the tests reach the error path)
+            if (const char* e = getenv("TURBOFFT_FUSED_LIMIT_MS")) if (atoi(e) != 0) q->pair_limit_ms = atoi(e);
+            if (const char* e = getenv("TURBOFFT_FUSED_PROF")) q->pair_prof = atoi(e) != 0;
             if (q->pair_teams_per_xcd < 1 || q->pair_teams_per_xcd > 64) { turbofft_plan_destroy(q); break; }   // no room for a team: the plan keeps its two launches
             p->pair = q;
             if (!pair_add_ws(p, q, nullptr, false)) { turbofft_plan_destroy(q); p->pair = nullptr; return fail(TURBOFFT_ENOMEM, "no memory for the slots of the fused pair"); }
@@ -1290,12 +1297,7 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         f.team = p->pair_team;
         f.teams_per_xcd = p->pair_teams_per_xcd;
         f.limit_ms = p->pair_limit_ms;
-        if (getenv("TURBOFFT_FUSED_PROF")) {
-            // diagnostic (kernels built with TFFT_PAIR_PROFILE set): time per part of a round, printed per execution
-            static unsigned long long* prof = nullptr;
-            if (!prof) { if (hipMalloc((void**)&prof, 8 * sizeof(unsigned long long) * 65536) != hipSuccess) prof = nullptr; }
-            f.prof = prof;
-        }
+        f.prof = w->prof;          // diagnostic builds of the kernel only (TFFT_PAIR_PROFILE at build time) write it
         if (f.npieces > 0x7fffffffll) return fail(TURBOFFT_EINVAL, "too many pieces for the fused kernel");
         const void* in_arg = in_d;
         void* out_arg = out;
@@ -1304,7 +1306,9 @@ static int exec_impl(turbofft_plan_t* p, const void* in_d, void* out_d, long lon
         HIP_TRY(hipLaunchKernel(p->pk->func, dim3((unsigned)p->pair_grid), dim3((unsigned)p->pk->threads), args, (size_t)p->pk->lds_bytes,
                                 (hipStream_t)stream));
         if (o.sync_each) HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        if (f.prof && getenv("TURBOFFT_FUSED_PROF") && atoi(getenv("TURBOFFT_FUSED_PROF")) == 2) {
+        if (f.prof && !stream_is_capturing(stream)) {
+            // TURBOFFT_FUSED_PROF=1 when the plan was made: wait for the execution and print what a diagnostic build of the
+            // kernel timed (ticks of 10 ns per block and part of a round; all zero from a product build)
             HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
             std::vector<unsigned long long> h((size_t)8 * p->pair_grid);
             HIP_TRY(hipMemcpy(h.data(), f.prof, h.size() * 8, hipMemcpyDeviceToHost));
