@@ -259,7 +259,7 @@ def test_delayed_batch_correction_host_chosen_tiles_and_earlier_launch():
     plan.close()
 
 
-COMPACT = [("float2", 7, 4096), ("float2", 9, 1024), ("float2", 13, 64), ("float2", 14, 32), ("float2", 15, 16), ("float2", 19, 2), ("float2", 20, 2), ("float2", 22, 1), ("double2", 7, 4096)]
+COMPACT = [("float2", 7, 4096), ("float2", 9, 1024), ("float2", 13, 64), ("float2", 14, 32), ("float2", 15, 16), ("float2", 19, 2), ("float2", 20, 2), ("float2", 22, 1), ("float2", 23, 1), ("double2", 7, 4096)]
 
 
 @pytest.mark.parametrize("dt,logN,bs", COMPACT)
@@ -639,7 +639,7 @@ def test_groups_shared_by_several_blocks(dt, logN, bs, tbs):
 
 TL_CASES = [("float2", 10, 64), ("double2", 10, 16), ("float2", 13, 32), ("double2", 15, 8), ("float2", 16, 4),
             ("float2", 21, 1), ("double2", 20, 2), ("float2", 24, 1), ("float2", 5, 1000), ("double2", 3, 777),
-            ("float2", 15, 6), ("double2", 14, 5)]
+            ("float2", 15, 6), ("double2", 14, 5), ("float2", 23, 1)]
 
 
 @pytest.mark.parametrize("dt,logN,bs", TL_CASES)
