@@ -706,3 +706,63 @@ def test_thread_level_verification_in_an_earlier_launch_and_refusals():
     with pytest.raises(turbofft_amd.TurboFFTError):
         plan.set_checksum_mode("reference")                   # no table to choose
     plan.close()
+
+
+@pytest.mark.parametrize("dt", ["float2", "double2"])
+@pytest.mark.parametrize("logN", list(range(1, 25)))
+def test_checked_plans_of_every_size_run_clean(dt, logN):
+    # every row of the fault-tolerant and of the thread-level tables, the sizes no other case names included:
+    # a ragged batch of clean data gives the DFT, raises nothing, and every tile of every launch was checked
+    # (groups of four tiles walked by one block, groups of thirty-two shared by several, thread-level)
+    bs = (1 << max(0, 20 - logN)) + 3
+    x = make(bs, 1 << logN, dt, 700 + logN)
+    want = O.fft_ref(x)
+    for if_ft, tbs in ((1, 4), (1, 32), (2, 1)):
+        plan = turbofft_amd.TurboFFT(logN, dt, if_ft=if_ft, thread_bs=tbs)
+        y, c = run(plan, x)
+        assert c["detected"] == 0 and c["flagged"] == [], (if_ft, tbs, c)
+        assert O.rel_l2(y, want) <= O.tolerance(dt, logN), (if_ft, tbs)
+        geoms = O.launch_geometry(O.PlanRow.from_list(plan.plan_row()), bs)
+        if if_ft == 2:
+            assert c["checked"] == sum(g.ntiles for g in geoms)
+        else:
+            assert c["checked"] == sum(plan.grid(i, bs) for i in range(plan.launches))
+        plan.close()
+
+
+def _thread_level_rows():
+    import os
+    out = []
+    for dt in ("float2", "double2"):
+        path = os.path.join(os.path.dirname(turbofft_amd.__file__), "param", "gfx950", f"param_{dt}_tt.csv")
+        with open(path) as f:
+            out += [(dt, [int(v) for v in line.split(",")]) for line in f if line.strip() and not line.startswith("#")]
+    return out
+
+
+@pytest.mark.parametrize("dt,csv_row", _thread_level_rows(), ids=lambda v: v if isinstance(v, str) else f"2^{v[0]}")
+def test_thread_level_rows_of_their_own(dt, csv_row):
+    # every size whose thread-level plan runs a row of its own (param_<T>_tt.csv): the plan has that shape,
+    # clean data (a ragged batch) raises nothing and gives the DFT, one large error in one tile of the last
+    # launch is caught in exactly that tile, and the tile recomputed before it is stored leaves the result
+    # bit-identical to the undisturbed run
+    logN, L = csv_row[0], csv_row[1]
+    plan = turbofft_amd.TurboFFT(logN, dt, if_ft=2)
+    assert plan.launches == L and list(plan.logNi) == csv_row[2:2 + L] and list(plan.BS) == csv_row[5:5 + L] and list(plan.n) == csv_row[8:8 + L]
+    assert all(n.endswith("_tt") for n in plan.kernel_names()), plan.kernel_names()
+    bs = (1 << max(0, 21 - logN)) + 3
+    x = make(bs, 1 << logN, dt, 300 + logN)
+    plan.set_ft_params(1000.0, 1e-3, correct=1)
+    plan.set_injection(0)
+    y0, c0 = run(plan, x)
+    row = O.PlanRow.from_list(plan.plan_row())
+    geoms = O.launch_geometry(row, bs)
+    assert c0["detected"] == 0 and c0["checked"] == sum(g.ntiles for g in geoms)
+    assert O.rel_l2(y0, O.fft_ref(x)) <= O.tolerance(dt, logN)
+    last = L - 1
+    tile = min(5, geoms[last].ntiles - 1)
+    plan.set_injection(2, launch=last, every=1 << 30, tile_phase=tile, s=plan.BS[last] - 1, m=0, mag=1.0e6)
+    y, c = run(plan, x)
+    assert c["flagged"] == [(last, tile)] and c["detected"] == 1 == c["corrected"] and c["uncorrectable"] == 0
+    assert np.array_equal(y, y0)
+    plan.close()
