@@ -166,9 +166,10 @@ def test_prefetch_row1(kind, dtype, logNi, BS, n, split, tbs, pf):
     assert O.rel_l2(y, O.fft_ref(x.astype(simlib.ctype_of(dtype)))) < O.tolerance(dtype, logNi)
 
 
-def test_prefetch_col_and_rowT():
+@pytest.mark.parametrize("pf", [1, 3])
+def test_prefetch_col_and_rowT(pf):
     dtype = "float2"
-    sp = KernelSpec(KernelKey(dtype, "col", 8, 16, 16, 0, 0, 1))
+    sp = KernelSpec(KernelKey(dtype, "col", 8, 16, 16, 0, 0, pf))
     Ni, ncols, outer, log_ncols = 256, 64, 3, 6
     x = rnd((outer, Ni, ncols), 5)
     ka = simlib.KArgs()
@@ -179,7 +180,7 @@ def test_prefetch_col_and_rowT():
     ref = np.fft.fft(x.astype(np.complex64).astype(np.complex128), axis=1)
     ref = ref * np.exp(-2j * np.pi * ((np.arange(Ni)[:, None] * np.arange(ncols)[None, :]) % (Ni * ncols)) / (Ni * ncols))
     assert O.rel_l2(y, ref) < O.tolerance(dtype, 8)
-    sp = KernelSpec(KernelKey(dtype, "rowT", 8, 16, 16, 0, 0, 1))
+    sp = KernelSpec(KernelKey(dtype, "rowT", 8, 16, 16, 0, 0, pf))
     A, Q, Cc = 256, 2, 32
     x = rnd((2, Cc, Q, A), 7)
     ka = simlib.KArgs()

@@ -111,8 +111,8 @@ class KernelSpec:
         # pf > 1: only the first pf elements of a thread are fetched ahead, and only from the start
         # of the tile's last pass on (for 1024-thread blocks, which have no room for a whole set)
         self.pfk = int(k.pf) if int(k.pf) > 1 else 0
-        if self.pfk and (k.kind != "row1" or int(k.ft) or k.xl or self.pfk >= k.n or (k.BS == 1 and k.n and False)):
-            raise ValueError(f"{k}: partial prefetch is for plain single-launch kernels, fewer elements than n")
+        if self.pfk and (int(k.ft) or k.xl or self.pfk >= k.n):
+            raise ValueError(f"{k}: partial prefetch is for plain kernels, fewer elements than n")
         self.xl = bool(k.xl)        # last (radix 2/4/8) pass across lanes instead of through LDS
         self.lds_esize = self.esize // 2 if self.split else self.esize   # bytes per LDS access
         self.passes = radix_passes(self.Ni, self.n)
@@ -546,32 +546,19 @@ class KernelEmitter:
 
     def emit_load(self, c: Code, dst: str = "r", sfx: str = "", elems: Optional[Sequence[int]] = None):
         """Loads of a tile's elements into dst[e]; `elems` restricts them to some of a thread's
-        elements (row1 kernels, one element per access)."""
+        elements (one element per access, forward kernels)."""
         sp = self.s
         lNi = ilog2(sp.Ni)
+        pairs = self.pair_access() and elems is None
         if elems is not None:
-            assert sp.kind == "row1" and not self.pair_access() and not int(sp.key.inv)
-            c(f"const unsigned gi{sfx} = (s << {lNi}) + x;")
-            if sp.BS > 1:
-                c(f"if ((row0{sfx} + s) < a.nrows) {{")
-                c.ind += 1
-            for e in elems:
-                c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
-            if sp.BS > 1:
-                c.ind -= 1
-                c("} else {")
-                c.ind += 1
-                for e in elems:
-                    c(f"{dst}[{e}] = czero({dst}[0]);")
-                c.ind -= 1
-                c("}")
-            return
+            assert not self.pair_access() and not int(sp.key.inv)
+        es = list(elems) if elems is not None else list(range(sp.n))
         if sp.kind == "row1":
             c(f"const unsigned gi{sfx} = (s << {lNi}) + x;")
             if sp.BS > 1:
                 c(f"if ((row0{sfx} + s) < a.nrows) {{")
                 c.ind += 1
-            if self.pair_access():
+            if pairs:
                 # a buffer that starts on an odd element takes the one-element accesses (uniform branch)
                 c("if (((unsigned long long)in & 15ull) == 0ull) {")
                 c.ind += 1
@@ -580,26 +567,26 @@ class KernelEmitter:
                 c.ind -= 1
                 c("} else {")
                 c.ind += 1
-            for e in range(sp.n):
+            for e in es:
                 c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {sp.Tr * e}, gi{sfx});")
-            if self.pair_access():
+            if pairs:
                 c.ind -= 1
                 c("}")
             if sp.BS > 1:
                 c.ind -= 1
                 c("} else {")
                 c.ind += 1
-                for e in range(sp.n):
+                for e in es:
                     c(f"{dst}[{e}] = czero({dst}[0]);")
                 c.ind -= 1
                 c("}")
         elif sp.kind == "col":
             c(f"const unsigned gi{sfx} = s + (x << a.log_ncols);")
-            for e in range(sp.n):
+            for e in es:
                 c(f"{dst}[{e}] = {self.GLD}(in, ubase{sfx}, {e} * gstep{sfx}, gi{sfx});")
         else:
             c(f"const unsigned gi{sfx} = ((s << a.logQ) << {lNi}) + x;")
-            for e in range(sp.n):
+            for e in es:
                 c(f"{dst}[{e}] = {self.GLD}(in, {'ubase_ld' if self.role == 'B' else 'ubase_in'}{sfx}, {sp.Tr * e}, gi{sfx});")
         if int(sp.key.inv) and sp.kind in ("row1", "col"):
             # inverse plan, first launch: a forward transform of (im, re) is (im, re) of the
@@ -1043,6 +1030,9 @@ class KernelEmitter:
                     # is alone on its CU and would otherwise have nothing in flight while it computes
                     c("if (has_next) {")
                     c.ind += 1
+                    if sp.maps[q] != sp.maps[0]:
+                        # a tile is loaded with the thread map of its first pass (this scope's s and x)
+                        self.map_vars(c, 0)
                     self.emit_tile_decode(c, "tile_n", "_n")
                     self.emit_load(c, "rn", "_n", elems=range(sp.pfk))
                     c.ind -= 1
