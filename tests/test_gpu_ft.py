@@ -259,7 +259,7 @@ def test_delayed_batch_correction_host_chosen_tiles_and_earlier_launch():
     plan.close()
 
 
-COMPACT = [("float2", 7, 4096), ("float2", 9, 1024), ("float2", 13, 64), ("float2", 14, 32), ("float2", 15, 16), ("float2", 19, 2), ("float2", 20, 2), ("float2", 22, 1), ("float2", 23, 1), ("double2", 7, 4096), ("double2", 15, 16), ("double2", 20, 2), ("double2", 23, 1)]
+COMPACT = [("float2", 7, 4096), ("float2", 9, 1024), ("float2", 13, 64), ("float2", 14, 32), ("float2", 15, 16), ("float2", 16, 8), ("float2", 17, 4), ("float2", 18, 2), ("float2", 19, 2), ("float2", 20, 2), ("float2", 22, 1), ("float2", 23, 1), ("double2", 7, 4096), ("double2", 15, 16), ("double2", 20, 2), ("double2", 23, 1)]
 
 
 @pytest.mark.parametrize("dt,logN,bs", COMPACT)
